@@ -1,0 +1,116 @@
+"""Build libmi_gemm.so: render one HIP translation unit per kernel configuration from the
+Jinja templates, compile them for gfx950 in parallel with hipcc, link the C ABI.
+
+    python -m h100_gemm_amd.build [-j JOBS] [--force]
+
+Takes the place of the reference's `nvcc -arch=sm_90a ... -o test` line (Makefile:1-5 and
+gemm_tuner.py:46 in the reference tree).  Nothing here needs a GPU.
+"""
+from __future__ import annotations
+
+import argparse
+import hashlib
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+from jinja2 import Template
+
+from . import kernel_configs as kc
+
+PKG = Path(__file__).resolve().parent
+CSRC = PKG / "csrc"
+GEN = CSRC / "gen"
+LIB = PKG / "lib" / "libmi_gemm.so"
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+# -packed-fp32-ops off: packed fp32 VALU forms are not to be generated on this hardware pool.
+HIPFLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature",
+            "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
+            f"-I{CSRC}", f"-I{GEN}"]
+
+
+def _write_if_changed(path: Path, text: str) -> None:
+    if not path.exists() or path.read_text() != text:
+        path.write_text(text)
+
+
+def render_sources(configs=None) -> list[Path]:
+    """Render the per-config units and the kernel table; returns the units' paths."""
+    configs = kc.CONFIGS if configs is None else configs
+    GEN.mkdir(parents=True, exist_ok=True)
+    unit_t = Template((PKG / "template" / "kernel_unit.hip.jinja").read_text())
+    table_t = Template((PKG / "template" / "kernel_table.hpp.jinja").read_text())
+    named = [dict(c, name=kc.config_name(c)) for c in configs]
+    units = []
+    for c in named:
+        p = GEN / f"unit_{c['name']}.hip"
+        _write_if_changed(p, unit_t.render(**c))
+        units.append(p)
+    names = [c["name"] for c in named]
+    big = names.index(kc.config_name(kc.DEFAULT_BIG)) if hasattr(kc, "DEFAULT_BIG") else 0
+    small = names.index(kc.config_name(kc.DEFAULT_SMALL)) if hasattr(kc, "DEFAULT_SMALL") else len(names) - 1
+    _write_if_changed(GEN / "kernel_table.hpp",
+                      table_t.render(configs=named, big_index=big, small_index=small,
+                                     big_min_tiles=getattr(kc, "BIG_MIN_TILES", 64)))
+    # drop units of configs that no longer exist
+    keep = {p.name for p in units}
+    for old in GEN.glob("unit_*.hip"):
+        if old.name not in keep:
+            old.unlink()
+            old.with_suffix(".o").unlink(missing_ok=True)
+    return units
+
+
+def _stamp(src: Path) -> str:
+    h = hashlib.sha1()
+    for dep in [src, CSRC / "gemm_kernel.hpp", CSRC / "gemm_launch.hpp", GEN / "kernel_table.hpp",
+                PKG.parent / "include" / "mi_gemm.h"]:
+        h.update(dep.read_bytes())
+    h.update(" ".join(HIPFLAGS).encode())
+    return h.hexdigest()
+
+
+def _compile(src: Path, force: bool) -> Path:
+    obj = src.with_suffix(".o") if src.parent == GEN else GEN / (src.stem + ".o")
+    stamp = obj.with_suffix(".stamp")
+    want = _stamp(src)
+    if not force and obj.exists() and stamp.exists() and stamp.read_text() == want:
+        return obj
+    cmd = [HIPCC, *HIPFLAGS, "-c", str(src), "-o", str(obj)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {src.name}:\n{r.stderr[-4000:]}")
+    stamp.write_text(want)
+    return obj
+
+
+def build(jobs: int | None = None, force: bool = False, verbose: bool = True) -> Path:
+    units = render_sources()
+    srcs = units + [CSRC / "mi_gemm.hip", CSRC / "reference_gpu_gemm.hip"]
+    jobs = jobs or min(8, os.cpu_count() or 1)
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        objs = list(ex.map(lambda s: _compile(s, force), srcs))
+    LIB.parent.mkdir(parents=True, exist_ok=True)
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB), *map(str, objs)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"link failed:\n{r.stderr[-4000:]}")
+    if verbose:
+        print(f"built {LIB} ({LIB.stat().st_size} bytes, {len(units)} kernel configs)")
+    return LIB
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(description=__doc__)
+    ap.add_argument("-j", "--jobs", type=int, default=None)
+    ap.add_argument("--force", action="store_true")
+    a = ap.parse_args(argv)
+    build(a.jobs, a.force)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

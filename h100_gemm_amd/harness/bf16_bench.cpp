@@ -1,0 +1,98 @@
+// bf16_bench.cpp -- the benchmark program of the reference's bf16 kernel
+// (main() of matmul_h100_optimal.cu:115-229) on the MI355X library: N(0,1) bf16 inputs
+// from a default_random_engine(69), a verification pass that doubles as warm-up, then
+// `repeat_times` back-to-back launches between two events and the line
+//     Average elapsed time: (s) s, performance: (T) TFLOPS. size: (n).
+// Differences, all on purpose: the golden is the library's plain ascending-k GPU GEMM
+// instead of a vendor BLAS (kernel 0 of the reference), the comparison the reference left
+// disabled (`kernel_num > 1`, matmul_h100_optimal.cu:177) is enabled, its hard-coded 8192
+// index math is gone, the size can be given as `./bf16_bench [size] [repeats]`, and the
+// 5 s cool-down before each kernel (matmul_h100_optimal.cu:160) is behind `sleep 1` env
+// MI_BENCH_SLEEP.
+#include <unistd.h>
+
+#include "gemm_host.hpp"
+
+int main(int argc, char** argv) {
+    long max_size = argc > 1 ? std::atol(argv[1]) : 8192;
+    int repeat_times = argc > 2 ? std::atoi(argv[2]) : 8;
+    long m = max_size, n = max_size, k = max_size;
+    const size_t elems = (size_t)max_size * max_size;
+
+    float elapsed_time;
+    void *start, *stop;
+    MI_CHECK(mi_event_create(&start));
+    MI_CHECK(mi_event_create(&stop));
+
+    bf16* A = (bf16*)malloc(sizeof(bf16) * elems);
+    bf16* B = (bf16*)malloc(sizeof(bf16) * elems);
+    bf16* C = (bf16*)malloc(sizeof(bf16) * elems);
+    bf16* C_ref = (bf16*)malloc(sizeof(bf16) * elems);
+    randomize_matrix(A, elems);
+    randomize_matrix(B, elems);
+    randomize_matrix(C, elems);
+
+    const size_t db_words = mi_gemm_trace_words((int)m, (int)n, (int)k);
+    int* DB = (int*)malloc(sizeof(int) * db_words);
+    void *dA, *dB, *dC, *dC_ref, *dDB;
+    MI_CHECK(mi_malloc(&dA, sizeof(bf16) * elems));
+    MI_CHECK(mi_malloc(&dB, sizeof(bf16) * elems));
+    MI_CHECK(mi_malloc(&dC, sizeof(bf16) * elems));
+    MI_CHECK(mi_malloc(&dC_ref, sizeof(bf16) * elems));
+    MI_CHECK(mi_malloc(&dDB, sizeof(int) * db_words));
+    MI_CHECK(mi_memcpy_h2d(dA, A, sizeof(bf16) * elems));
+    MI_CHECK(mi_memcpy_h2d(dB, B, sizeof(bf16) * elems));
+
+    const char* sl = getenv("MI_BENCH_SLEEP");
+    for (int kernel_num : {1}) {
+        if (sl) sleep(std::atoi(sl));   // cool-down of matmul_h100_optimal.cu:160
+        std::cout << "KERNEL " << kernel_num << std::endl;
+        // verification, also the warm-up
+        memset(C, 0, sizeof(bf16) * elems);
+        MI_CHECK(mi_memcpy_h2d(dC, C, sizeof(bf16) * elems));
+        MI_CHECK(mi_memcpy_h2d(dC_ref, C, sizeof(bf16) * elems));
+        memset(DB, ~0, sizeof(int) * db_words);
+        MI_CHECK(mi_memcpy_h2d(dDB, DB, sizeof(int) * db_words));
+        MI_CHECK(mi_reference_gpu_gemm(MI_DTYPE_BF16, (int)m, (int)n, (int)k, dA, dB, dC_ref, 1.0f, 0.0f, nullptr));
+        run_kernel(kernel_num, (int)m, (int)n, (int)k, (bf16*)dA, (bf16*)dB, (bf16*)dC, (int*)dDB);
+        MI_CHECK(mi_device_sync());
+        MI_CHECK(mi_memcpy_d2h(C, dC, sizeof(bf16) * elems));
+        MI_CHECK(mi_memcpy_d2h(C_ref, dC_ref, sizeof(bf16) * elems));
+        if (!verify_matrix(C_ref, C, elems)) {
+            std::cout << "~~~~~~~~~~~~~~~~ Failed to pass the correctness verification against the "
+                         "reference GEMM. ~~~~~~~~~~~~~~~~" << std::endl;
+            return 1;
+        }
+        // trace records: (sumLoad, cntLoad, sumCompute, cntCompute, sumStore, cntStore) per
+        // workgroup until the ~0 sentinel (matmul_h100_optimal.cu:182-198)
+        MI_CHECK(mi_memcpy_d2h(DB, dDB, sizeof(int) * db_words));
+        size_t i = 0;
+        long sumLoad = 0, cntLoad = 0, sumCompute = 0, cntCompute = 0, sumStore = 0, cntStore = 0;
+        int times = 0;
+        while (i + 5 < db_words && DB[i] != ~0) {
+            sumLoad += DB[i], cntLoad += DB[i + 1];
+            sumCompute += DB[i + 2], cntCompute += DB[i + 3];
+            sumStore += DB[i + 4], cntStore += DB[i + 5];
+            i += 6;
+            times++;
+        }
+        if (times > 0)
+            printf("Load: %f, Compute: %f,  Store: %f, Datapoints: %d\n", (sumLoad + .0) / cntLoad,
+                   (sumCompute + .0) / cntCompute, (sumStore + .0) / cntStore, times);
+
+        MI_CHECK(mi_event_record(start, nullptr));
+        for (int j = 0; j < repeat_times; j++) run_kernel(kernel_num, (int)m, (int)n, (int)k, (bf16*)dA, (bf16*)dB, (bf16*)dC);
+        MI_CHECK(mi_event_record(stop, nullptr));
+        MI_CHECK(mi_event_sync(start));
+        MI_CHECK(mi_event_sync(stop));
+        MI_CHECK(mi_event_elapsed_ms(&elapsed_time, start, stop));
+
+        long flops = (2LL * m) * (n * k);
+        printf("Average elapsed time: (%7.6f) s, performance: (%7.1f) TFLOPS. size: (%ld).\n\n",
+               elapsed_time / 1000.0 / repeat_times, (repeat_times * flops * 1e-9) / elapsed_time, m);
+    }
+
+    free(A); free(B); free(C); free(C_ref); free(DB);
+    mi_free(dA); mi_free(dB); mi_free(dC); mi_free(dC_ref); mi_free(dDB);
+    return 0;
+}

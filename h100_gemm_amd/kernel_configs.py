@@ -1,0 +1,72 @@
+"""The kernel configurations compiled into libmi_gemm.so.
+
+Each entry fixes the template constants of ``csrc/gemm_kernel.hpp`` -- the counterpart of the
+six constants ``CLUSTER_M, CLUSTER_N, BLOCKM, BLOCKN, BLOCKK, STAGES`` that the reference's
+template takes (matmul_h100.cu.jinja:9-14) -- re-cast for CDNA4:
+
+    BM, BN   macro tile of one workgroup (the K step is fixed at 64 = one 128-byte LDS row)
+    WM, WN   wave grid: WM*WN waves of 64 lanes, each owning a (BM/WM) x (BN/WN) sub-tile
+    SWZ      LDS chunk swizzle (0: row & 7, 1: (row >> 1) & 7)
+    GROUP    tile-order group height (L2 locality of the workgroups sharing an XCD)
+    OCC      workgroups per CU the register budget is sized for
+
+The index of a config in ``CONFIGS`` is its ``config`` number in the C ABI.
+"""
+from __future__ import annotations
+
+
+def config_name(c: dict) -> str:
+    return (f"t{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_s{c['SWZ']}_g{c['GROUP']}"
+            f"_o{c['OCC']}")
+
+
+def lds_bytes(c: dict) -> int:
+    return 2 * (c["BM"] + c["BN"]) * 128
+
+
+def is_valid_config(c: dict) -> bool:
+    """Static rules of gemm_kernel.hpp (mirrored as static_asserts there)."""
+    nt = c["WM"] * c["WN"] * 64
+    if nt > 1024 or nt < 64:
+        return False
+    if c["BM"] % (32 * c["WM"]) or c["BN"] % (32 * c["WN"]):
+        return False
+    if (c["BM"] * 8) % nt or (c["BN"] * 8) % nt or (nt // 8) % 16:
+        return False
+    if lds_bytes(c) * c["OCC"] > 160 * 1024:
+        return False
+    mi, ni = c["BM"] // c["WM"] // 32, c["BN"] // c["WN"] // 32
+    nmma = mi * ni
+    if mi + ni > nmma or c["BM"] * 8 // nt > nmma or c["BN"] * 8 // nt > nmma:
+        return False
+    # accumulators (16 regs per 32x32 tile) + fragments + staging must fit 512 / waves-per-SIMD
+    waves_per_simd = max(nt // 256, 1) * c["OCC"]
+    regs = nmma * 16 + 2 * (mi + ni) * 4 + (c["BM"] + c["BN"]) * 8 // nt * 4 + 40
+    return regs <= 512 // waves_per_simd
+
+
+def _c(BM, BN, WM, WN, SWZ=1, GROUP=8, OCC=1):
+    return dict(BM=BM, BN=BN, WM=WM, WN=WN, SWZ=SWZ, GROUP=GROUP, OCC=OCC)
+
+
+CONFIGS = [
+    _c(256, 256, 2, 2, SWZ=1, GROUP=8),
+    _c(256, 256, 2, 2, SWZ=0, GROUP=8),
+    _c(256, 256, 2, 2, SWZ=1, GROUP=4),
+    _c(256, 256, 2, 2, SWZ=1, GROUP=16),
+    _c(256, 256, 2, 4, SWZ=1, GROUP=8),
+    _c(256, 256, 4, 2, SWZ=1, GROUP=8),
+    _c(256, 128, 2, 2, SWZ=1, GROUP=8),
+    _c(128, 256, 2, 2, SWZ=1, GROUP=8),
+    _c(128, 128, 2, 2, SWZ=1, GROUP=8, OCC=2),
+    _c(128, 128, 2, 2, SWZ=0, GROUP=8, OCC=2),
+]
+
+assert all(is_valid_config(c) for c in CONFIGS), [config_name(c) for c in CONFIGS if not is_valid_config(c)]
+assert len({config_name(c) for c in CONFIGS}) == len(CONFIGS)
+
+# What MI_CONFIG_AUTO resolves to: the big tile when there are enough 256x256 tiles to
+# occupy the chip, the small one otherwise.
+DEFAULT_BIG = CONFIGS[0]
+DEFAULT_SMALL = CONFIGS[8]
+BIG_MIN_TILES = 64

@@ -1,0 +1,123 @@
+/*
+ * mi_gemm.h -- C ABI of the MI355X (gfx950) dense GEMM library, libmi_gemm.so.
+ *
+ *     C[M,N] = A[M,K] . B[N,K]^T      16-bit float storage, fp32 accumulate (MFMA)
+ *
+ * A is M x K row-major, B is N x K row-major ("K-major"), C is M x N row-major; leading
+ * dimensions are K, K and N.  All matrix pointers are DEVICE pointers owned by the
+ * caller.  Launches are asynchronous on the given HIP stream (NULL = the null stream) and
+ * C is fully overwritten (no read of C, beta = 0, alpha = 1), which is what the launchers
+ * this library replaces do.
+ *
+ * Each entry point cites the host function of the reference project (Faraz9877/H100_GEMM)
+ * whose place it takes.  The reference has no FFI: its boundary is a handful of host C++
+ * functions linked into one executable; `h100_gemm_amd/harness/gemm_host.hpp` rebuilds
+ * those functions (same names, same arguments, same exit-on-error behaviour) as inline
+ * shims over this ABI.
+ *
+ * Every function returning int returns 0 on success and a negative MI_ERR_* code on
+ * failure; mi_last_error() then holds a message for the calling thread.
+ */
+#ifndef MI_GEMM_H
+#define MI_GEMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI_OK 0
+#define MI_ERR_INVALID (-1) /* bad shape, null pointer, unknown config or dtype */
+#define MI_ERR_HIP (-2)     /* a HIP runtime call failed; see mi_last_error()   */
+#define MI_ERR_UNSUPPORTED (-3) /* the chosen kernel config cannot run this shape */
+
+#define MI_DTYPE_BF16 0
+#define MI_DTYPE_FP16 1
+
+#define MI_CONFIG_AUTO (-1)
+
+/* ---- the GEMM ---------------------------------------------------------------------- */
+
+/* bf16 GEMM with the library's own choice of kernel for the shape.
+ * Replaces  void runKernel(int M, int N, int K, bf16* A, bf16* B, bf16* C, int* DB)
+ * (matmul_h100_optimal.cu:32-59) and the `case 1` arm of run_kernel
+ * (matmul_h100_optimal.cu:75-84).  DB may be NULL; when it is not, it is the device
+ * trace buffer of that signature (see mi_gemm_trace_words()). */
+int mi_gemm_bf16(int M, int N, int K, const uint16_t* A, const uint16_t* B, uint16_t* C,
+                 int* DB, void* stream);
+
+/* The same GEMM with an explicit kernel configuration and storage type.
+ * Replaces  template<...> void gpu_gemm<AType,BType,CType,AccumType,CLUSTER_M,CLUSTER_N,
+ * BLOCKM,BLOCKN,BLOCKK,STAGES>(GemmParams)  (matmul_h100.cu.jinja:927-985): the template
+ * arguments of that launcher become `config` (an index into the table below, or
+ * MI_CONFIG_AUTO) and `dtype` (MI_DTYPE_*). */
+int mi_gemm_ex(int config, int dtype, int M, int N, int K, const void* A, const void* B,
+               void* C, int* DB, void* stream);
+
+/* Plain, order-preserving GPU GEMM used as golden by the harness: one fp32 accumulator per
+ * element fed in ascending k, C = (CType)(acc * alpha + beta), beta a scalar.
+ * Replaces  reference_gpu_gemm(GemmParams)  (reference.h:78-90), which the reference's
+ * harness compares its kernel with (matmul_h100.cu.jinja:1043-1047). */
+int mi_reference_gpu_gemm(int dtype, int M, int N, int K, const void* A, const void* B, void* C,
+                          float alpha, float beta, void* stream);
+
+/* Kernel configuration table (what the tuner sweeps; replaces the six template constants
+ * of matmul_h100.cu.jinja:9-14). */
+int mi_gemm_num_configs(void);
+/* Human-readable name, e.g. "t256x256x64_w2x2_rs1_sw1_g8"; NULL if out of range. */
+const char* mi_gemm_config_name(int config);
+/* Index of the config with that name, or -1. */
+int mi_gemm_find_config(const char* name);
+/* The config MI_CONFIG_AUTO resolves to for this shape (never negative for valid shapes). */
+int mi_gemm_select_config(int dtype, int M, int N, int K);
+/* 1 if `config` can run this shape (alignment / divisibility rules of that kernel). */
+int mi_gemm_config_supports(int config, int dtype, int M, int N, int K);
+/* Workgroups and static LDS bytes the config launches for this shape (0 if unsupported). */
+int mi_gemm_config_grid(int config, int M, int N, int K);
+int mi_gemm_config_lds_bytes(int config);
+
+/* Number of `int` words a DB trace buffer must hold for this shape so that the kernel's
+ * per-workgroup records plus the terminating sentinel fit (the harness of
+ * matmul_h100_optimal.cu:132-139 allocates 8192*128 ints). */
+size_t mi_gemm_trace_words(int M, int N, int K);
+
+/* ---- thin HIP layer used by the C++ harness ------------------------------------------
+ * These stand where the reference's harness calls the CUDA runtime directly
+ * (common.h:309-365 alloc/copy/free, common.h:246-273 GPUTimer, common.h:43-60
+ * get_sm_count, matmul_h100_optimal.cu:120-122,203-210 events). */
+int mi_malloc(void** dptr, size_t bytes);
+int mi_free(void* dptr);
+int mi_memcpy_h2d(void* dst, const void* src, size_t bytes);
+int mi_memcpy_d2h(void* dst, const void* src, size_t bytes);
+int mi_memset(void* dst, int value, size_t bytes);
+int mi_device_sync(void);
+int mi_stream_sync(void* stream);
+int mi_event_create(void** ev);
+int mi_event_destroy(void* ev);
+int mi_event_record(void* ev, void* stream);
+int mi_event_sync(void* ev);
+int mi_event_elapsed_ms(float* ms, void* start, void* stop);
+
+typedef struct mi_device_props {
+    char name[256];
+    char arch[64];
+    int compute_units;       /* what get_sm_count() returns on the reference side */
+    int clock_khz;           /* peak engine clock */
+    int mem_clock_khz;
+    int mem_bus_bits;
+    int lds_bytes_per_block; /* max LDS one workgroup may use */
+    int l2_bytes;
+    int wavefront;
+    size_t hbm_bytes;
+} mi_device_props;
+int mi_get_device_props(mi_device_props* out);
+
+/* Message of the last failure on this thread ("" if none). */
+const char* mi_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI_GEMM_H */
