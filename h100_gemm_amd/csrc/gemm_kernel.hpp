@@ -62,13 +62,17 @@ struct GemmArgs {
 //   SWZ          LDS chunk swizzle: 0 -> row & 7, 1 -> (row >> 1) & 7
 //   GROUP        height, in tiles, of the column-major groups of the tile order
 //   OCC          workgroups per CU the register / LDS budget is sized for
+//   DTL          1: global -> LDS by direct-to-LDS buffer loads (no staging registers, no
+//                ds_write); 0: global -> registers -> ds_write.  The predicated variant
+//                always stages through registers (it has to mask the K tail there).
 //   EDGE         predicated variant: any M, N, K and any alignment
 //   DT           storage type (DT_BF16 / DT_FP16)
-template <int BM_, int BN_, int WM_, int WN_, int SWZ_, int GROUP_, int OCC_, bool EDGE_, int DT_>
+template <int BM_, int BN_, int WM_, int WN_, int SWZ_, int GROUP_, int OCC_, int DTL_, bool EDGE_, int DT_>
 struct TileConfig {
     static constexpr int BM = BM_, BN = BN_, BK = 64;
     static constexpr int WM = WM_, WN = WN_;
     static constexpr int SWZ = SWZ_, GROUP = GROUP_, OCC = OCC_;
+    static constexpr bool DTL = DTL_ != 0 && !EDGE_;
     static constexpr bool EDGE = EDGE_;
     static constexpr int DT = DT_;
     static constexpr int NT = WM * WN * 64;             // threads per workgroup
@@ -139,10 +143,21 @@ __device__ __forceinline__ void tile_of_block(int pid, int nwg, int tiles_m, int
     tn = in / gsz;
 }
 
-template <class Cfg>
+// TRACE = true adds the per-workgroup timing record the reference's bf16 harness knows how
+// to read from its `int* DB` argument (matmul_h100_optimal.cu:182-198): six ints
+//   { sumLoad, cntLoad, sumCompute, cntCompute, sumStore, cntStore }
+// at DB[6 * blockIdx.x], in s_memtime ticks: Load = time wave 0 spent at the per-K-step
+// barrier (waiting for operands to land and for the other waves), counted once per K step;
+// Compute = the whole main loop, counted per K step; Store = the epilogue, counted once.
+// The caller pre-fills DB with ~0 so the first unused word terminates the list.
+template <class Cfg, bool TRACE = false>
 __global__ void __launch_bounds__(Cfg::NT)
 __attribute__((amdgpu_waves_per_eu(Cfg::WAVES_PER_EU, Cfg::WAVES_PER_EU)))
 gemm_tile_kernel(const GemmArgs p) {
+    long long tr_wait = 0, tr_t0 = 0, tr_loop = 0;
+    int tr_cnt = 0;
+    auto tr_now = [&]() __attribute__((always_inline)) { return (long long)__builtin_readcyclecounter(); };
+    if constexpr (TRACE) tr_loop = tr_now();
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
     constexpr int WN = Cfg::WN;
     constexpr int MI = Cfg::MI, NI = Cfg::NI, LA = Cfg::LA, LB = Cfg::LB;
@@ -295,105 +310,234 @@ gemm_tile_kernel(const GemmArgs p) {
                 acc[i][j] = mfma_32x32x16<DT>(fb[buf][j], fa[buf][i], acc[i][j]);
     };
 
-    // ---- prologue: tile 0 -> LDS stage 0, tile 1 -> registers ----
-    gload_a(0);
-    gload_b(0);
-    if constexpr (EDGE) mask_tail(0);
-    lds_store_a(0);
-    lds_store_b(0);
-    gload_a(1);
-    gload_b(1);
-    lds_barrier();
-    read_frags(0, 0, 0);
-
-    // One K step = four 16-deep k slices (ks), 16 MFMAs each for a 128x128 wave tile.
-    // LDS[cur] holds tile kt, registers hold tile kt+1 (if any).
-    //   ks 0 : MFMA(ks 0) | fetch fragments ks 1 | A registers (tile kt+1) -> LDS[nxt]
-    //   ks 1 : MFMA(ks 1) | fetch fragments ks 2 | B registers -> LDS[nxt], global loads of
-    //          A for tile kt+2
-    //   ks 2 : MFMA(ks 2) | fetch fragments ks 3 | global loads of B for tile kt+2
-    //   barrier: LDS[nxt] complete, LDS[cur] drained
-    //   ks 3 : MFMA(ks 3) | fetch fragments ks 0 of tile kt+1 from LDS[nxt]
-    // Every write to a stage follows the barrier that ended the step in which it was last
-    // read, and every read follows the barrier after it was written: one barrier per step.
-    // The sched_group_barrier sequences ask the scheduler to deal the memory instructions
-    // of a slice out between its MFMAs instead of bunching them in front.
-    auto interleave = [&](auto nmfma_c, auto nread_c, auto nwrite_c, auto nvmem_c) __attribute__((always_inline)) {
-        constexpr int nmfma = decltype(nmfma_c)::value, nread = decltype(nread_c)::value;
-        constexpr int nwrite = decltype(nwrite_c)::value, nvmem = decltype(nvmem_c)::value;
+    if constexpr (Cfg::DTL) {
+        // ---- direct-to-LDS pipeline (aligned shapes) ----
+        // A buffer load with the `lds` modifier writes lane l's 16 bytes to LDS address
+        // M0 + 16*l, so one wave instruction fills 8 consecutive 128-byte rows.  The LDS
+        // swizzle is therefore applied on the global side: the lane that lands on chunk
+        // position c' of row r fetches logical chunk c' ^ swz(r).  Wave w, pass j fills
+        // rows (j*NW + w)*8 .. +7 of the tile.
+        // The compiler knows nothing of these loads (they are inline asm), so the waits on
+        // them are explicit: vmcnt(0) before the barrier that publishes a stage.
+        const int lr = lane >> 3, lc = lane & 7;
+        const int drow = wave * 8 + lr;                       // tile row of pass 0
+        const int dchunk = lc ^ swz(drow);
+        const uint32_t dvoffA = (uint32_t)(drow * p.lda + dchunk * 8) * 2u;
+        const uint32_t dvoffB = (uint32_t)(drow * p.ldb + dchunk * 8) * 2u;
+        const uint32_t lds_base =
+            (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
+        const uint32_t dlds = lds_base + (uint32_t)wave * 1024u;   // + stage + pass * RPP * 128
+        auto dma = [&](const __amdgpu_buffer_rsrc_t& rsrc, uint32_t voff, uint32_t dst) __attribute__((always_inline)) {
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                         :: "s"(dst), "v"(voff), "s"(rsrc) : "memory");
+        };
+        auto dma_a = [&](int kt, int stage) __attribute__((always_inline)) {
+            const uint32_t kb = (uint32_t)kt * (BK * 2);
 #pragma unroll
-        for (int i = 0; i < nmfma; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);              // one MFMA
-            if (i < nread) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
-            if (i >= nmfma - nwrite) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // LDS write
-            if (i >= nmfma - nvmem) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // global load
+            for (int j = 0; j < LA; ++j)
+                dma(rsrcA, dvoffA + kb + j * passA, dlds + stage * A_STAGE + j * (RPP * 128));
+        };
+        auto dma_b = [&](int kt, int stage) __attribute__((always_inline)) {
+            const uint32_t kb = (uint32_t)kt * (BK * 2);
+#pragma unroll
+            for (int j = 0; j < LB; ++j)
+                dma(rsrcB, dvoffB + kb + j * passB, dlds + 2 * A_STAGE + stage * B_STAGE + j * (RPP * 128));
+        };
+        auto vm_barrier = [&]() __attribute__((always_inline)) {
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        };
+        constexpr int NMMA = MI * NI, NFR = MI + NI;
+        constexpr int DPM = (LA + LB + NMMA - 1) / NMMA;     // DMA instructions per MFMA slot
+        // One MFMA, in the order (i, j) = (idx / NI, idx % NI).
+        auto mma_one = [&](int buf, int idx) __attribute__((always_inline)) {
+            const int i = idx / NI, j = idx % NI;
+            acc[i][j] = mfma_32x32x16<DT>(fb[buf][j], fa[buf][i], acc[i][j]);
+        };
+        // Fragment r of a k slice, in the order the MFMAs above first need them:
+        // A0, B0, B1, .., B(NI-1), A1, .., A(MI-1).
+        auto read_one = [&](int stage, int ks, int buf, int r) __attribute__((always_inline)) {
+            if (r == 0 || r > NI) {
+                const int i = r == 0 ? 0 : r - NI;
+                fa[buf][i] = *(const u32x4_t*)(lds + stage * A_STAGE + a_wave + i * 4096 + rd_off[ks]);
+            } else {
+                const int j = r - 1;
+                fb[buf][j] = *(const u32x4_t*)(lds + 2 * A_STAGE + stage * B_STAGE + b_wave + j * 4096 + rd_off[ks]);
+            }
+        };
+        auto dma_one = [&](int kt, int stage, int d) __attribute__((always_inline)) {
+            const uint32_t kb = (uint32_t)kt * (BK * 2);
+            if (d < LA)
+                dma(rsrcA, dvoffA + kb + d * passA, dlds + stage * A_STAGE + d * (RPP * 128));
+            else if (d < LA + LB)
+                dma(rsrcB, dvoffB + kb + (d - LA) * passB,
+                    dlds + 2 * A_STAGE + stage * B_STAGE + (d - LA) * (RPP * 128));
+        };
+        // tile 0 -> stage 0, tile 1 -> stage 1
+        dma_a(0, 0);
+        dma_b(0, 0);
+        dma_a(1, 1);
+        dma_b(1, 1);
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"(LA + LB) : "memory");   // tile 0 landed
+#pragma unroll
+        for (int r = 0; r < NFR; ++r) read_one(0, 0, 0, r);
+        // One K step.  LDS[cur] = tile kt, LDS[nxt] = tile kt+1 (landing).
+        //   ks 0..2 : MFMA | fetch fragments ks+1 from LDS[cur]
+        //   vmcnt(0) + barrier : tile kt+1 complete, LDS[cur] drained by every wave
+        //   ks 3    : MFMA | fetch fragments ks 0 of tile kt+1 | start tile kt+2 -> LDS[cur]
+        // Each slot is pinned (one MFMA, then at most one LDS read and DPM loads) so the
+        // memory instructions are dealt out between the MFMAs.
+        auto dstep = [&](int kt, auto cur_c, auto has1_c, auto has2_c) __attribute__((always_inline)) {
+            constexpr int cur = decltype(cur_c)::value;
+            constexpr int nxt = cur ^ 1;
+            constexpr bool has1 = decltype(has1_c)::value;
+            constexpr bool has2 = decltype(has2_c)::value;
+#pragma unroll
+            for (int ks = 0; ks < 3; ++ks) {
+#pragma unroll
+                for (int idx = 0; idx < NMMA; ++idx) {
+                    mma_one(ks & 1, idx);
+                    if (idx < NFR) read_one(cur, ks + 1, (ks + 1) & 1, idx);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            if constexpr (has1) {
+                if constexpr (TRACE) tr_t0 = tr_now();
+                vm_barrier();
+                if constexpr (TRACE) { tr_wait += tr_now() - tr_t0; ++tr_cnt; }
+            }
+#pragma unroll
+            for (int idx = 0; idx < NMMA; ++idx) {
+                mma_one(1, idx);
+                if constexpr (has1) {
+                    if (idx < NFR) read_one(nxt, 0, 0, idx);
+                }
+                if constexpr (has2) {
+#pragma unroll
+                    for (int d = 0; d < DPM; ++d) dma_one(kt + 2, cur, idx * DPM + d);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        using T = std::true_type;
+        using F = std::false_type;
+        using S0 = std::integral_constant<int, 0>;
+        using S1 = std::integral_constant<int, 1>;
+        int kt = 0;
+        for (; kt + 2 < KT; kt += 2) {
+            dstep(kt, S0{}, T{}, T{});
+            dstep(kt + 1, S1{}, T{}, T{});
         }
-    };
-    constexpr int NMMA = MI * NI, NFR = MI + NI;
-    static_assert(NFR <= NMMA && LA <= NMMA && LB <= NMMA, "interleave pattern assumes it");
-    using I0 = std::integral_constant<int, 0>;
-    using IM = std::integral_constant<int, NMMA>;
-    using IR = std::integral_constant<int, NFR>;
-    using IA = std::integral_constant<int, LA>;
-    using IB = std::integral_constant<int, LB>;
-    auto kstep = [&](int kt, auto cur_c, auto has1_c, auto has2_c, auto mask_c) __attribute__((always_inline)) {
-        constexpr bool mask = decltype(mask_c)::value;   // tile kt+1 may cross K
-        constexpr int cur = decltype(cur_c)::value;
-        constexpr int nxt = cur ^ 1;
-        constexpr bool has1 = decltype(has1_c)::value;   // tile kt+1 exists
-        constexpr bool has2 = decltype(has2_c)::value;   // tile kt+2 exists
-        // ks 0
-        read_frags(cur, 1, 1);
-        if constexpr (has1) {
-            if constexpr (mask) mask_tail(kt + 1);
-            lds_store_a(nxt);
-        }
-        mma(0);
-        if constexpr (has1) interleave(IM{}, IR{}, IA{}, I0{}); else interleave(IM{}, IR{}, I0{}, I0{});
-        __builtin_amdgcn_sched_barrier(0);
-        // ks 1
-        read_frags(cur, 2, 0);
-        if constexpr (has1) lds_store_b(nxt);
-        if constexpr (has2) gload_a(kt + 2);
-        mma(1);
-        if constexpr (has2) interleave(IM{}, IR{}, IB{}, IA{});
-        else if constexpr (has1) interleave(IM{}, IR{}, IB{}, I0{});
-        else interleave(IM{}, IR{}, I0{}, I0{});
-        __builtin_amdgcn_sched_barrier(0);
-        // ks 2
-        read_frags(cur, 3, 1);
-        if constexpr (has2) gload_b(kt + 2);
-        mma(0);
-        if constexpr (has2) interleave(IM{}, IR{}, I0{}, IB{}); else interleave(IM{}, IR{}, I0{}, I0{});
-        __builtin_amdgcn_sched_barrier(0);
+        dstep(kt, S0{}, T{}, F{});
+        dstep(kt + 1, S1{}, F{}, F{});
+    } else {
+        // ---- prologue: tile 0 -> LDS stage 0, tile 1 -> registers ----
+        gload_a(0);
+        gload_b(0);
+        if constexpr (EDGE) mask_tail(0);
+        lds_store_a(0);
+        lds_store_b(0);
+        gload_a(1);
+        gload_b(1);
         lds_barrier();
-        // ks 3
-        if constexpr (has1) read_frags(nxt, 0, 0);
-        mma(1);
-        if constexpr (has1) interleave(IM{}, IR{}, I0{}, I0{});
-        __builtin_amdgcn_sched_barrier(0);
-    };
-    using T = std::true_type;
-    using F = std::false_type;
-    using S0 = std::integral_constant<int, 0>;
-    using S1 = std::integral_constant<int, 1>;
-    // Steady state, two steps per trip; then the draining steps.  Only the last two tiles
-    // can cross K (KT is rounded up to even), so only the steps that move those tiles into
-    // LDS carry the masking code.
-    using E = std::integral_constant<bool, EDGE>;
-    int kt = 0;
-    for (; kt + 4 < KT; kt += 2) {
-        kstep(kt, S0{}, T{}, T{}, F{});
-        kstep(kt + 1, S1{}, T{}, T{}, F{});
-    }
-    if (KT >= 4) {
-        kstep(kt, S0{}, T{}, T{}, F{});
-        kstep(kt + 1, S1{}, T{}, T{}, E{});
-        kt += 2;
-    }
-    kstep(kt, S0{}, T{}, F{}, E{});
-    kstep(kt + 1, S1{}, F{}, F{}, F{});
+        read_frags(0, 0, 0);
 
+        // One K step = four 16-deep k slices (ks), 16 MFMAs each for a 128x128 wave tile.
+        // LDS[cur] holds tile kt, registers hold tile kt+1 (if any).
+        //   ks 0 : MFMA(ks 0) | fetch fragments ks 1 | A registers (tile kt+1) -> LDS[nxt]
+        //   ks 1 : MFMA(ks 1) | fetch fragments ks 2 | B registers -> LDS[nxt], global loads of
+        //          A for tile kt+2
+        //   ks 2 : MFMA(ks 2) | fetch fragments ks 3 | global loads of B for tile kt+2
+        //   barrier: LDS[nxt] complete, LDS[cur] drained
+        //   ks 3 : MFMA(ks 3) | fetch fragments ks 0 of tile kt+1 from LDS[nxt]
+        // Every write to a stage follows the barrier that ended the step in which it was last
+        // read, and every read follows the barrier after it was written: one barrier per step.
+        // The sched_group_barrier sequences ask the scheduler to deal the memory instructions
+        // of a slice out between its MFMAs instead of bunching them in front.
+        auto interleave = [&](auto nmfma_c, auto nread_c, auto nwrite_c, auto nvmem_c) __attribute__((always_inline)) {
+            constexpr int nmfma = decltype(nmfma_c)::value, nread = decltype(nread_c)::value;
+            constexpr int nwrite = decltype(nwrite_c)::value, nvmem = decltype(nvmem_c)::value;
+    #pragma unroll
+            for (int i = 0; i < nmfma; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);              // one MFMA
+                if (i < nread) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+                if (i >= nmfma - nwrite) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // LDS write
+                if (i >= nmfma - nvmem) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // global load
+            }
+        };
+        constexpr int NMMA = MI * NI, NFR = MI + NI;
+        static_assert(NFR <= NMMA && LA <= NMMA && LB <= NMMA, "interleave pattern assumes it");
+        using I0 = std::integral_constant<int, 0>;
+        using IM = std::integral_constant<int, NMMA>;
+        using IR = std::integral_constant<int, NFR>;
+        using IA = std::integral_constant<int, LA>;
+        using IB = std::integral_constant<int, LB>;
+        auto kstep = [&](int kt, auto cur_c, auto has1_c, auto has2_c, auto mask_c) __attribute__((always_inline)) {
+            constexpr bool mask = decltype(mask_c)::value;   // tile kt+1 may cross K
+            constexpr int cur = decltype(cur_c)::value;
+            constexpr int nxt = cur ^ 1;
+            constexpr bool has1 = decltype(has1_c)::value;   // tile kt+1 exists
+            constexpr bool has2 = decltype(has2_c)::value;   // tile kt+2 exists
+            // ks 0
+            read_frags(cur, 1, 1);
+            if constexpr (has1) {
+                if constexpr (mask) mask_tail(kt + 1);
+                lds_store_a(nxt);
+            }
+            mma(0);
+            if constexpr (has1) interleave(IM{}, IR{}, IA{}, I0{}); else interleave(IM{}, IR{}, I0{}, I0{});
+            __builtin_amdgcn_sched_barrier(0);
+            // ks 1
+            read_frags(cur, 2, 0);
+            if constexpr (has1) lds_store_b(nxt);
+            if constexpr (has2) gload_a(kt + 2);
+            mma(1);
+            if constexpr (has2) interleave(IM{}, IR{}, IB{}, IA{});
+            else if constexpr (has1) interleave(IM{}, IR{}, IB{}, I0{});
+            else interleave(IM{}, IR{}, I0{}, I0{});
+            __builtin_amdgcn_sched_barrier(0);
+            // ks 2
+            read_frags(cur, 3, 1);
+            if constexpr (has2) gload_b(kt + 2);
+            mma(0);
+            if constexpr (has2) interleave(IM{}, IR{}, I0{}, IB{}); else interleave(IM{}, IR{}, I0{}, I0{});
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (TRACE) tr_t0 = tr_now();
+            lds_barrier();
+            if constexpr (TRACE) { tr_wait += tr_now() - tr_t0; ++tr_cnt; }
+            // ks 3
+            if constexpr (has1) read_frags(nxt, 0, 0);
+            mma(1);
+            if constexpr (has1) interleave(IM{}, IR{}, I0{}, I0{});
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        using T = std::true_type;
+        using F = std::false_type;
+        using S0 = std::integral_constant<int, 0>;
+        using S1 = std::integral_constant<int, 1>;
+        // Steady state, two steps per trip; then the draining steps.  Only the last two tiles
+        // can cross K (KT is rounded up to even), so only the steps that move those tiles into
+        // LDS carry the masking code.
+        using E = std::integral_constant<bool, EDGE>;
+        int kt = 0;
+        for (; kt + 4 < KT; kt += 2) {
+            kstep(kt, S0{}, T{}, T{}, F{});
+            kstep(kt + 1, S1{}, T{}, T{}, F{});
+        }
+        if (KT >= 4) {
+            kstep(kt, S0{}, T{}, T{}, F{});
+            kstep(kt + 1, S1{}, T{}, T{}, E{});
+            kt += 2;
+        }
+        kstep(kt, S0{}, T{}, F{}, E{});
+        kstep(kt + 1, S1{}, F{}, F{}, F{});
+
+    }
+
+    long long tr_store = 0;
+    if constexpr (TRACE) {
+        tr_store = tr_now();
+        tr_loop = tr_store - tr_loop;
+    }
     // ---- epilogue: fp32 -> storage type, 8-byte stores into row-major C ----
     // acc[i][j][e] of lane l is C[m][n] with m = row of A fragment = l & 31,
     // n = 8*(e/4) + 4*(l>>5) + (e%4) inside the 32x32 tile.
@@ -433,6 +577,19 @@ gemm_tile_kernel(const GemmArgs p) {
                     }
                 }
             }
+        }
+    }
+    if constexpr (TRACE) {
+        if (p.DB != nullptr && tid == 0) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the stores have left the wave
+            tr_store = tr_now() - tr_store;
+            int* rec = p.DB + 6 * (size_t)blockIdx.x;
+            rec[0] = (int)tr_wait;
+            rec[1] = tr_cnt;
+            rec[2] = (int)tr_loop;
+            rec[3] = KT;
+            rec[4] = (int)tr_store;
+            rec[5] = 1;
         }
     }
 }

@@ -115,8 +115,13 @@ int mi_gemm_select_config(int dtype, int M, int N, int K) {
 }
 
 size_t mi_gemm_trace_words(int M, int N, int K) {
-    int cfg = mi::select_kernel(M, N, K);
-    return (size_t)mi_gemm_config_grid(cfg, M, N, K) * 6 + 1;
+    // enough for whichever kernel configuration ends up running the shape
+    size_t grid = 0;
+    for (int c = 0; c < mi::kNumKernels; ++c) {
+        const size_t g = (size_t)mi_gemm_config_grid(c, M, N, K);
+        if (g > grid) grid = g;
+    }
+    return grid * 6 + 1;
 }
 
 int mi_gemm_ex(int config, int dtype, int M, int N, int K, const void* A, const void* B,

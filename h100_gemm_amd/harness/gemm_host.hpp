@@ -221,6 +221,42 @@ void constant_fill(DType* tensor, std::vector<int> shape, DType value) {
     for (size_t i = 0; i < length; ++i) tensor[i] = value;
 }
 
+// Seeded, counter-based fills used for the benchmark configurations: element i of stream s
+// is a pure function of (seed, s, i), so the same matrices can be regenerated anywhere.
+// (The reference's own generators are unseeded rand() and a library-defined
+// std::normal_distribution; these are this library's additions.)
+inline uint64_t mi_mix64(uint64_t z) {
+    z += 0x9e3779b97f4a7c15ull;
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+    return z ^ (z >> 31);
+}
+inline uint64_t mi_rng_u64(uint64_t seed, uint64_t stream, uint64_t index) {
+    return mi_mix64(mi_mix64(seed ^ (stream * 0xd1342543de82ef95ull)) + index);
+}
+// i.i.d. uniform on the 2^-23 grid of [-1, 1), rounded to the storage type.
+template <class DType>
+void uniform_fill(DType* tensor, std::vector<int> shape, uint64_t seed, uint64_t stream) {
+    const size_t length = shape_numel(shape);
+    for (size_t i = 0; i < length; ++i) {
+        const float u = (float)(mi_rng_u64(seed, stream, i) >> 40) * (1.0f / 16777216.0f);
+        tensor[i] = DType(2.0f * u - 1.0f);
+    }
+}
+// i.i.d. N(0, sigma^2) by Box-Muller in double, rounded once to the storage type.
+template <class DType>
+void normal_fill(DType* tensor, std::vector<int> shape, uint64_t seed, uint64_t stream,
+                 float sigma = 1.0f) {
+    const size_t length = shape_numel(shape);
+    for (size_t i = 0; i < length; ++i) {
+        const uint64_t r = mi_rng_u64(seed, stream, i);
+        const double u1 = ((double)(r >> 40) + 1.0) * (1.0 / 16777216.0);
+        const double u2 = (double)(r & 0xffffffull) * (1.0 / 16777216.0);
+        const double z = std::sqrt(-2.0 * std::log(u1)) * std::cos(6.283185307179586476925 * u2);
+        tensor[i] = DType((float)(z * (double)sigma));
+    }
+}
+
 template <class DType>
 DType* alloc_gpu_tensor(std::vector<int> shape) {
     void* dt;
