@@ -328,6 +328,9 @@ gemm_tile_kernel(const GemmArgs p) {
             (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
         const uint32_t dlds = lds_base + (uint32_t)wave * 1024u;   // + stage + pass * RPP * 128
         auto dma = [&](const __amdgpu_buffer_rsrc_t& rsrc, uint32_t voff, uint32_t dst) __attribute__((always_inline)) {
+#ifdef MI_EXP_NO_DMA
+            if (K > 0) return;
+#endif
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                          :: "s"(dst), "v"(voff), "s"(rsrc) : "memory");
         };
@@ -346,6 +349,8 @@ gemm_tile_kernel(const GemmArgs p) {
         auto vm_barrier = [&]() __attribute__((always_inline)) {
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
         };
+        int kt_dbg = 0;
+        (void)kt_dbg;
         constexpr int NMMA = MI * NI, NFR = MI + NI;
         constexpr int DPM = (LA + LB + NMMA - 1) / NMMA;     // DMA instructions per MFMA slot
         // One MFMA, in the order (i, j) = (idx / NI, idx % NI).
@@ -356,6 +361,9 @@ gemm_tile_kernel(const GemmArgs p) {
         // Fragment r of a k slice, in the order the MFMAs above first need them:
         // A0, B0, B1, .., B(NI-1), A1, .., A(MI-1).
         auto read_one = [&](int stage, int ks, int buf, int r) __attribute__((always_inline)) {
+#ifdef MI_EXP_NO_READS
+            if (kt_dbg > 1) return;
+#endif
             if (r == 0 || r > NI) {
                 const int i = r == 0 ? 0 : r - NI;
                 fa[buf][i] = *(const u32x4_t*)(lds + stage * A_STAGE + a_wave + i * 4096 + rd_off[ks]);
@@ -391,6 +399,7 @@ gemm_tile_kernel(const GemmArgs p) {
             constexpr int nxt = cur ^ 1;
             constexpr bool has1 = decltype(has1_c)::value;
             constexpr bool has2 = decltype(has2_c)::value;
+            kt_dbg = kt;
 #pragma unroll
             for (int ks = 0; ks < 3; ++ks) {
 #pragma unroll

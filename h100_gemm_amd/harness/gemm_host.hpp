@@ -390,3 +390,33 @@ inline bool verify_matrix(bf16* matRef, bf16* matOut, size_t N) {
     }
     return true;
 }
+
+// The acceptance test of this library's benchmark configurations (not a reference
+// function): every element must satisfy
+//     |out - ref| <= 2^-7 * |ref| + 1e-3 * sqrt(K) * max|a| * max|b|.
+// verify_matrix's absolute 0.1 is tighter than one bf16 unit in the last place once
+// |C| >= 16, so two correct fp32-accumulating GEMMs that sum in different orders fail it
+// at the benchmark sizes; the reference leaves it disabled (matmul_h100_optimal.cu:177).
+// Returns the number of violating elements and prints the first one.
+template <class DType>
+inline size_t verify_tolerance(const DType* ref, const DType* out, size_t n, int K, double max_a,
+                               double max_b) {
+    const double abs_term = 1e-3 * std::sqrt((double)K) * max_a * max_b;
+    size_t bad = 0;
+    for (size_t i = 0; i < n; ++i) {
+        const double r = (float)ref[i], o = (float)out[i];
+        const double err = std::fabs(o - r);
+        if (!(err <= std::fabs(r) / 128.0 + abs_term)) {
+            if (bad == 0)
+                printf("Divergence! Should %5.2f, Is %5.2f (Diff %5.2f) at %zu\n", r, o, err, i);
+            ++bad;
+        }
+    }
+    return bad;
+}
+template <class DType>
+inline double max_abs_value(const DType* x, size_t n) {
+    double m = 0.0;
+    for (size_t i = 0; i < n; ++i) m = std::max(m, (double)std::fabs((float)x[i]));
+    return m;
+}

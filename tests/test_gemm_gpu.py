@@ -1,0 +1,254 @@
+"""Parity of the gfx950 kernels with the CPU oracle, through the C ABI (libmi_gemm.so).
+
+Tolerance (floating point, stated by the benchmark definition): per element
+    |out - ref| <= 2^-7 * |ref| + 1e-3 * sqrt(K) * max|a| * max|b|
+with `ref` the oracle's restatement of reference_cpu_gemm on the same seeded inputs.  With
+the reference's integer random_fill every partial sum is an exact integer, so there the
+bar is bit-exact.  Full-size shapes are compared on a fixed sample of 64x64 tiles (every
+tile of reference.h is independent, so a sampled tile holds exactly the full run's values)
+plus size-independent properties (row/column permutation equivariance, identity, run-to-run
+determinism).
+"""
+import re
+import subprocess
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+ROOT = Path(__file__).resolve().parent.parent
+
+
+class Dev:
+    """Device copies of A, B and an output buffer; frees on exit."""
+
+    def __init__(self, mi, A, B, M, N, pad=0):
+        self.mi, self.M, self.N, self.pad = mi, M, N, pad
+        self.dA = mi.DeviceBuffer.from_numpy(A)
+        self.dB = mi.DeviceBuffer.from_numpy(B)
+        self.dC = mi.DeviceBuffer(M * N * 2 + 64)
+        self.dC.fill_bytes(0xFF)
+
+    def run(self, K, config=-1, dtype=0, DB=None):
+        p = self.mi.GemmParams(self.M, self.N, K, self.dA, self.dB, self.dC)
+        self.mi.gpu_gemm(p, config=config, dtype=dtype, DB=DB)
+        self.mi.synchronize()
+        return self.dC.to_numpy((self.M, self.N), np.uint16)
+
+
+def make_inputs(orc, M, N, K, fill, dtype=0, seed=69):
+    if fill == "uniform":
+        return orc.fill_uniform((M, K), seed, 1, dtype), orc.fill_uniform((N, K), seed, 2, dtype)
+    if fill == "normal":      # activations N(0,1), weights N(0, 0.02^2)
+        return orc.fill_normal((M, K), seed, 1, 1.0, dtype), orc.fill_normal((N, K), seed, 2, 0.02, dtype)
+    if fill == "int":
+        return orc.fill_randint((M, K), seed, 1, dtype), orc.fill_randint((N, K), seed, 2, dtype)
+    raise ValueError(fill)
+
+
+def check(mi, orc, M, N, K, fill, config=-1, dtype=0, tiles=None, exact=False):
+    print(f"case M={M} N={N} K={K} fill={fill} config={config} dtype={dtype}", flush=True)
+    A, B = make_inputs(orc, M, N, K, fill, dtype)
+    C = Dev(mi, A, B, M, N).run(K, config, dtype)
+    ref = orc.reference_cpu_gemm(A, B, dtype=dtype, tiles=tiles)
+    rep = orc.check_tolerance(C, ref, K, orc.max_abs(A, dtype), orc.max_abs(B, dtype), dtype, tiles=tiles)
+    assert rep["violations"] == 0, rep
+    assert rep["compared"] > 0
+    if exact:
+        assert tiles is None
+        assert (C == ref).all(), f"{int((C != ref).sum())} elements differ"
+    return C, ref, rep
+
+
+# ---------------------------------------------------------------- benchmark configs ----
+
+def test_c1_square_512(mi, orc):
+    check(mi, orc, 512, 512, 512, "uniform")
+
+
+def test_c2_square_8192_sampled_tiles(mi, orc):
+    tiles = orc.sample_tiles(8192, 8192, 192)
+    check(mi, orc, 8192, 8192, 8192, "uniform", tiles=tiles)
+
+
+@pytest.mark.parametrize("M,N,K", [(8192, 28672, 8192), (8192, 8192, 28672)])
+def test_c3_mlp_shapes_sampled_tiles(mi, orc, M, N, K):
+    tiles = orc.sample_tiles(M, N, 96)
+    check(mi, orc, M, N, K, "normal", tiles=tiles)
+
+
+@pytest.mark.parametrize("M", [16, 64, 128])
+def test_c4_skinny_full(mi, orc, M):
+    check(mi, orc, M, 8192, 8192, "normal")
+
+
+def test_c5_unaligned_full(mi, orc):
+    check(mi, orc, 4095, 6143, 3073, "uniform")
+
+
+# ------------------------------------------------------ every kernel configuration ----
+
+def all_configs():
+    from h100_gemm_amd import kernel_configs as kc
+    return list(range(len(kc.CONFIGS)))
+
+
+@pytest.mark.parametrize("config", all_configs())
+def test_every_config_bit_exact_on_integer_fill(mi, orc, config):
+    # aligned (512^3: the aligned kernel), and ragged M, N, odd K (the predicated kernel)
+    for M, N, K in [(512, 512, 512), (768, 1280, 1152), (257, 515, 77), (300, 200, 136)]:
+        check(mi, orc, M, N, K, "int", config=config, exact=True)
+
+
+@pytest.mark.parametrize("config", all_configs())
+def test_every_config_uniform_within_tolerance(mi, orc, config):
+    for M, N, K in [(1024, 768, 256), (255, 511, 129)]:
+        check(mi, orc, M, N, K, "uniform", config=config)
+
+
+# --------------------------------------------------------------------- edge cases ----
+
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (1, 1, 64), (1, 300, 7), (300, 1, 9), (2, 3, 1),
+                                   (64, 64, 63), (65, 63, 65), (129, 127, 128), (256, 256, 127),
+                                   (256, 256, 2048), (31, 33, 4097), (1000, 1000, 8)])
+def test_ragged_and_tiny_shapes(mi, orc, M, N, K):
+    check(mi, orc, M, N, K, "int", exact=True)
+    check(mi, orc, M, N, K, "uniform")
+
+
+def test_k_tail_with_page_aligned_matrix_end(mi, orc):
+    # odd K with M a multiple of 2048: the last element of A sits right below a 4 KiB
+    # boundary of the allocation; the kernel must fetch it without reading past the matrix
+    check(mi, orc, 2048, 96, 77, "int", exact=True)
+    check(mi, orc, 96, 2048, 65, "int", exact=True)
+
+
+def test_misaligned_base_pointers(mi, orc):
+    # sub-matrices that start 2 bytes into an allocation: nothing is 16-byte aligned
+    M, N, K = 200, 264, 160
+    A, B = make_inputs(orc, M, N, K, "int")
+    ref = orc.reference_cpu_gemm(A, B)
+    dA = mi.DeviceBuffer(A.nbytes + 16)
+    dB = mi.DeviceBuffer(B.nbytes + 16)
+    dC = mi.DeviceBuffer(M * N * 2 + 16)
+    L = mi._lib.load()
+    mi._lib.check(L.mi_memcpy_h2d(dA.ptr + 2, A.ctypes.data, A.nbytes))
+    mi._lib.check(L.mi_memcpy_h2d(dB.ptr + 6, B.ctypes.data, B.nbytes))
+    dC.fill_bytes(0xEE)
+    mi.runKernel(M, N, K, dA.ptr + 2, dB.ptr + 6, dC.ptr + 2)
+    mi.synchronize()
+    raw = dC.to_numpy((M * N + 8,), np.uint16)
+    assert (raw[1:1 + M * N].reshape(M, N) == ref).all()
+    assert raw[0] == 0xEEEE and (raw[1 + M * N:] == 0xEEEE).all()      # nothing written outside C
+
+
+def test_output_buffer_is_not_overrun(mi, orc):
+    M, N, K = 257, 515, 77
+    A, B = make_inputs(orc, M, N, K, "int")
+    d = Dev(mi, A, B, M, N)
+    d.run(K)
+    tail = d.dC.to_numpy((M * N + 32,), np.uint16)[M * N:]
+    assert (tail == 0xFFFF).all()
+
+
+def test_fp16_storage(mi, orc):
+    for M, N, K in [(512, 512, 512), (130, 70, 200)]:
+        check(mi, orc, M, N, K, "int", dtype=orc.FP16, exact=True)
+        check(mi, orc, M, N, K, "uniform", dtype=orc.FP16)
+
+
+def test_known_answer_fills(mi, orc):
+    # constant_fill / arange_fill closed forms (common.h:292-307)
+    M, N, K = 256, 256, 256
+    A = orc.fill_constant((M, K), 0.5)
+    B = orc.fill_constant((N, K), 2.0)
+    C = Dev(mi, A, B, M, N).run(K)
+    assert (orc.to_f32(C) == 256.0).all()
+    A = orc.fill_arange((M, K), bound=16)
+    want = np.array([sum((i * K + k) % 16 for k in range(K)) for i in range(M)], dtype=np.float32)
+    C = Dev(mi, A, orc.fill_constant((N, K), 1.0), M, N).run(K)
+    assert (C == orc.from_f32(np.repeat(want[:, None], N, 1))).all()
+    # identity: I . B^T = B^T exactly
+    eye = orc.from_f32(np.eye(256, dtype=np.float32))
+    Bu = orc.fill_uniform((384, 256), 5, 2)
+    assert (Dev(mi, eye, Bu, 256, 384).run(256) == Bu.T).all()
+
+
+# ------------------------------------------------------- properties at full size ------
+
+def test_full_size_permutation_equivariance_and_determinism(mi, orc):
+    M = N = K = 8192
+    A, B = make_inputs(orc, M, N, K, "uniform")
+    d = Dev(mi, A, B, M, N)
+    C0 = d.run(K)
+    assert (d.run(K) == C0).all()                         # run-to-run bit identical
+    rng = np.random.default_rng(3)
+    pm, pn = rng.permutation(M), rng.permutation(N)
+    C1 = Dev(mi, A[pm], B[pn], M, N).run(K)
+    assert (C1 == C0[pm][:, pn]).all()                    # element values do not depend on tile
+    # zero K tail: K columns of zeros appended change nothing
+    Ah = np.concatenate([A[:, :4096], np.zeros((M, 64), np.uint16)], axis=1)
+    Bh = np.concatenate([B[:, :4096], np.zeros((N, 64), np.uint16)], axis=1)
+    Ca = Dev(mi, np.ascontiguousarray(A[:, :4096]), np.ascontiguousarray(B[:, :4096]), M, N).run(4096)
+    Cb = Dev(mi, Ah, Bh, M, N).run(4160)
+    assert (Ca == Cb).all()
+
+
+# ----------------------------------------------------- the harness's GPU golden -------
+
+def test_reference_gpu_gemm_is_bit_identical_to_the_oracle(mi, orc):
+    # same ascending-k fp32 accumulation, so not merely close: identical
+    for M, N, K, fill in [(300, 200, 517, "uniform"), (64, 64, 64, "normal"), (1, 5, 3, "uniform")]:
+        A, B = make_inputs(orc, M, N, K, fill)
+        dA, dB = mi.DeviceBuffer.from_numpy(A), mi.DeviceBuffer.from_numpy(B)
+        dC = mi.DeviceBuffer(M * N * 2)
+        mi.reference_gpu_gemm(mi.GemmParams(M, N, K, dA, dB, dC, 1.0, 0.0))
+        mi.synchronize()
+        assert (dC.to_numpy((M, N), np.uint16) == orc.reference_cpu_gemm(A, B)).all()
+        mi.reference_gpu_gemm(mi.GemmParams(M, N, K, dA, dB, dC, 0.5, 0.25))   # scalar beta
+        mi.synchronize()
+        assert (dC.to_numpy((M, N), np.uint16) == orc.reference_cpu_gemm(A, B, alpha=0.5, beta=0.25)).all()
+
+
+# ------------------------------------------------------------------ trace buffer ------
+
+def test_db_trace_records(mi, orc):
+    M = N = K = 1024
+    A, B = make_inputs(orc, M, N, K, "int")
+    d = Dev(mi, A, B, M, N)
+    words = mi._lib.load().mi_gemm_trace_words(M, N, K)
+    dDB = mi.DeviceBuffer(words * 4)
+    dDB.fill_bytes(0xFF)
+    cfg = mi.select_config(M, N, K)
+    C = d.run(K, DB=dDB)
+    assert (C == orc.reference_cpu_gemm(A, B)).all()        # tracing must not change results
+    db = dDB.to_numpy((words,), np.int32)
+    n = 0
+    while n + 5 < words and db[n] != -1:
+        n += 6
+    rec = db[:n].reshape(-1, 6)
+    assert len(rec) == mi.config_grid(cfg, M, N, K)
+    assert (rec[:, 3] == K // 64).all() and (rec[:, 5] == 1).all()
+    assert (rec[:, 2] > 0).all() and (rec[:, 0] >= 0).all() and (rec[:, 0] < rec[:, 2]).all()
+    assert db[n] == -1
+
+
+# --------------------------------------------------------------- C++ harness ----------
+
+def test_harness_programs(mi):
+    h = ROOT / "h100_gemm_amd" / "harness"
+    if not (h / "test").exists():
+        pytest.fail("harness programs are not built (make -C h100_gemm_amd/harness)")
+    r = subprocess.run([str(h / "test"), "M", "640", "N", "384", "K", "512", "iters", "5"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "Shape M=640, N=384, K=512" in r.stdout and "Correct!" in r.stdout
+    assert re.search(r"Average latency \(ms\) is ([\d.]+)", r.stdout)        # the tuner's regex
+    r = subprocess.run([str(h / "test"), "M", "333", "N", "129", "K", "77", "iters", "2",
+                        "dtype", "fp16"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0 and "Correct!" in r.stdout, r.stdout + r.stderr
+    r = subprocess.run([str(h / "bf16_bench"), "1024", "4"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "KERNEL 1" in r.stdout
+    assert re.search(r"Average elapsed time: \(\s*[\d.]+\) s, performance: \(\s*[\d.]+\) TFLOPS\. size: \(1024\)\.", r.stdout)

@@ -1,0 +1,178 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports every symbol that
+include/mi_gemm.h declares, argument validation happens before any device call, the Python
+mirror of the reference's host functions behaves like them, the kernel configuration table
+is consistent, and the tile-order mapping used by the kernels is a bijection."""
+import ctypes
+import itertools
+import re
+import subprocess
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+HEADER = ROOT / "include" / "mi_gemm.h"
+
+
+def declared_functions():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(mi_[a-z0-9_]+)\s*\(", text)) - {"mi_device_props"})
+
+
+def test_library_exports_every_declared_symbol(mi):
+    from h100_gemm_amd import _lib
+    names = declared_functions()
+    assert len(names) >= 20
+    lib = ctypes.CDLL(str(_lib.LIB_PATH))
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in mi_gemm.h but not exported"
+    assert set(names) == set(_lib.SYMBOLS), set(names) ^ set(_lib.SYMBOLS)
+
+
+def test_missing_library_fails_loudly(mi, monkeypatch, tmp_path):
+    from h100_gemm_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", tmp_path / "libmi_gemm.so")
+    with pytest.raises(ImportError, match="no fallback"):
+        _lib.load()
+
+
+def test_product_does_not_touch_the_oracle():
+    # the oracle is test infrastructure: nothing under the package may import, link or read it
+    for p in (ROOT / "h100_gemm_amd").rglob("*"):
+        if p.suffix in {".py", ".hpp", ".hip", ".cpp", ".jinja", ".h"} or p.name == "Makefile":
+            if "gen" in p.parts:
+                continue
+            text = p.read_text(errors="ignore")
+            assert not re.search(r"\boracle\b", text), f"{p} mentions the oracle"
+
+
+def test_argument_validation_needs_no_device(mi):
+    L = mi._lib.load()
+    bf = mi.MI_DTYPE_BF16
+    assert L.mi_gemm_bf16(0, 8, 8, 1, 1, 1, None, None) == mi._lib.MI_ERR_INVALID
+    assert b"positive" in L.mi_last_error()
+    assert L.mi_gemm_bf16(8, 8, 8, None, 1, 1, None, None) == mi._lib.MI_ERR_INVALID
+    assert L.mi_gemm_ex(999, bf, 8, 8, 8, 1, 1, 1, None, None) == mi._lib.MI_ERR_INVALID
+    assert L.mi_gemm_ex(-1, 7, 8, 8, 8, 1, 1, 1, None, None) == mi._lib.MI_ERR_INVALID
+    assert L.mi_gemm_ex(-1, bf, 70000, 70000, 8, 1, 1, 1, None, None) == mi._lib.MI_ERR_INVALID
+    assert L.mi_reference_gpu_gemm(bf, 8, -1, 8, 1, 1, 1, 1.0, 0.0, None) == mi._lib.MI_ERR_INVALID
+    with pytest.raises(mi.MiGemmError):
+        mi.runKernel(8, 8, 0, 1, 1, 1)
+    with pytest.raises(ValueError):
+        mi.run_kernel(0, 8, 8, 8, 1, 1, 1)          # 0 = vendor BLAS in the reference
+    with pytest.raises(ValueError):
+        mi.gpu_gemm(mi.GemmParams(8, 8, 8, 1, 1, 1, alpha=2.0))
+    with pytest.raises(ValueError):
+        mi.gpu_gemm(mi.GemmParams(8, 8, 8, 1, 1, 1), config="no_such_config")
+    with pytest.raises(TypeError):
+        mi.runKernel(8, 8, 8, "x", 1, 1)
+
+
+def test_config_table(mi):
+    from h100_gemm_amd import kernel_configs as kc
+    n = mi.num_configs()
+    assert n == len(kc.CONFIGS) >= 4
+    names = [mi.config_name(i) for i in range(n)]
+    assert names == [kc.config_name(c) for c in kc.CONFIGS]
+    assert mi.config_name(n) is None and mi.config_name(-1) is None
+    for i, nm in enumerate(names):
+        assert mi.find_config(nm) == i
+    assert mi.find_config("nope") == -1
+    L = mi._lib.load()
+    for i, c in enumerate(kc.CONFIGS):
+        assert L.mi_gemm_config_lds_bytes(i) == kc.lds_bytes(c) <= 160 * 1024
+        assert kc.is_valid_config(c)
+        tiles = -(-1000 // c["BM"]) * -(-777 // c["BN"])
+        assert mi.config_grid(i, 1000, 777, 64) == tiles
+        assert L.mi_gemm_config_supports(i, 0, 4095, 6143, 3073) == 1
+    assert mi.config_grid(0, 0, 8, 8) == 0
+    # the automatic choice is a valid index for every benchmark shape
+    for M, N, K in [(512, 512, 512), (8192, 8192, 8192), (8192, 28672, 8192), (8192, 8192, 28672),
+                    (16, 8192, 8192), (64, 8192, 8192), (128, 8192, 8192), (4095, 6143, 3073)]:
+        assert 0 <= mi.select_config(M, N, K) < n
+        assert L.mi_gemm_trace_words(M, N, K) >= 7
+    assert not kc.is_valid_config(dict(BM=256, BN=256, WM=2, WN=2, SWZ=1, GROUP=8, OCC=2, DTL=0))
+    assert not kc.is_valid_config(dict(BM=96, BN=256, WM=2, WN=2, SWZ=1, GROUP=8, OCC=1, DTL=0))
+
+
+def tile_of_block(pid, nwg, tiles_m, tiles_n, group):
+    """Python model of mi::tile_of_block (gemm_kernel.hpp)."""
+    q, r = nwg >> 3, nwg & 7
+    x, loc = pid & 7, pid >> 3
+    logical = x * q + min(x, r) + loc
+    gw = group * tiles_n
+    gid = logical // gw
+    first = gid * group
+    gsz = min(tiles_m - first, group)
+    inn = logical - gid * gw
+    return first + inn % gsz, inn // gsz
+
+
+def test_tile_order_is_a_bijection():
+    for tm, tn, g in itertools.product([1, 2, 3, 7, 16, 24, 32, 33], [1, 2, 5, 24, 32, 112], [1, 4, 8, 16]):
+        nwg = tm * tn
+        seen = {tile_of_block(p, nwg, tm, tn, g) for p in range(nwg)}
+        assert len(seen) == nwg and all(0 <= a < tm and 0 <= b < tn for a, b in seen)
+    # XCD locality: the 128 workgroups that land on XCD 0 of an 8192^2 launch (ids 0, 8, 16, ..)
+    # own a compact 8 x 16 block of tiles
+    tiles = {tile_of_block(p, 1024, 32, 32, 8) for p in range(0, 1024, 8)}
+    rows = {t[0] for t in tiles}
+    cols = {t[1] for t in tiles}
+    assert len(rows) == 8 and len(cols) == 16
+
+
+def test_harness_header_is_plain_host_cxx(tmp_path):
+    # gemm_host.hpp must compile with a host compiler alone (no HIP headers) and keep the
+    # reference's names and signatures usable
+    src = tmp_path / "t.cpp"
+    src.write_text(r'''
+#include "h100_gemm_amd/harness/gemm_host.hpp"
+int main() {
+    std::vector<int> s = {2, 3};
+    bf16* a = alloc_cpu_tensor<bf16>(s);
+    random_fill(a, s); arange_fill(a, s); constant_fill(a, s, bf16(1.5f));
+    GemmParams<bf16, bf16, bf16, float> p(2, 2, 3, a, a, a, 1.0f, 0.0f);
+    void (*f1)(int, int, int, bf16*, bf16*, bf16*, int*) = runKernel;
+    void (*f2)(int, int, int, int, bf16*, bf16*, bf16*, int*) = run_kernel;
+    (void)f1; (void)f2; (void)p;
+    CPUTimer t; t.tick(); t.tick(); (void)t.report_last_ms();
+    float x = (float)bf16(1.00390625f);      // tie -> even
+    float y = (float)half_t(65520.0f);       // overflow -> inf
+    free_cpu_tensor(a);
+    return (x == 1.0f && std::isinf(y) && (float)a[0] == (float)a[0]) ? 0 : 1;
+}
+''')
+    exe = tmp_path / "t"
+    r = subprocess.run(["g++", "-std=c++17", "-O1", f"-I{ROOT}", str(src), "-o", str(exe),
+                        f"-L{ROOT}/h100_gemm_amd/lib", "-lmi_gemm",
+                        f"-Wl,-rpath,{ROOT}/h100_gemm_amd/lib"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert subprocess.run([str(exe)]).returncode == 0
+
+
+def test_harness_fills_match_the_oracle(orc, tmp_path):
+    # the harness' seeded fills (product side, C++) and the oracle's (C) are two
+    # implementations of the same generators: same bits
+    src = tmp_path / "f.cpp"
+    src.write_text(r'''
+#include <cstdio>
+#include "h100_gemm_amd/harness/gemm_host.hpp"
+int main() {
+    std::vector<int> s = {4096};
+    std::vector<bf16> u(4096), n(4096);
+    uniform_fill(u.data(), s, 69, 1); normal_fill(n.data(), s, 69, 2, 0.02f);
+    fwrite(u.data(), 2, 4096, stdout); fwrite(n.data(), 2, 4096, stdout);
+    return 0;
+}
+''')
+    exe = tmp_path / "f"
+    r = subprocess.run(["g++", "-std=c++17", "-O1", f"-I{ROOT}", str(src), "-o", str(exe),
+                        f"-L{ROOT}/h100_gemm_amd/lib", "-lmi_gemm",
+                        f"-Wl,-rpath,{ROOT}/h100_gemm_amd/lib"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    raw = subprocess.run([str(exe)], capture_output=True).stdout
+    got = np.frombuffer(raw, dtype=np.uint16)
+    assert (got[:4096] == orc.fill_uniform((4096,), 69, 1)).all()
+    assert (got[4096:] == orc.fill_normal((4096,), 69, 2, 0.02)).all()
