@@ -1,0 +1,173 @@
+#!/usr/bin/env python3
+"""bench.py -- headline benchmark: bf16 GEMM TFLOP/s at M=N=K=8192 on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--config NAME]
+
+One "step" is one launch of the GEMM (A 8192x8192 row-major, B 8192x8192 K-major, both
+U[-1,1) seeded bf16, C bf16, fp32 accumulate) with the inputs already resident in HBM.
+Prints ONE JSON line.  `value` = 2*M*N*K / time per launch, in TFLOP/s.  The `roofline`
+object prices the kernel against MI355X's published dense bf16 MFMA peak (2.5 PFLOP/s);
+for the HBM-bound skinny workloads it is priced against 8 TB/s instead.  `cpu_baseline` is
+the CPU restatement of the reference's reference_cpu_gemm (reference.h:5-46) timed on this
+box's host cores on a bounded sample of 64x64 output tiles of the same problem.
+
+The timed region is bracketed by device synchronisation and measured with HIP events
+recorded on the stream the kernel is launched on (the null stream, as the reference's
+launchers use).  The library is loaded from h100_gemm_amd/lib; there is no fallback path.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+PEAK_BF16_TFLOPS = 2500.0     # MI355X published dense bf16 MFMA peak
+PEAK_HBM_GBS = 8000.0         # MI355X published HBM3E bandwidth
+
+# name -> (M, N, K, fill); fills as in the benchmark definition
+WORKLOADS = {
+    "square512": (512, 512, 512, "uniform"),
+    "square8192": (8192, 8192, 8192, "uniform"),
+    "mlp_up": (8192, 28672, 8192, "normal"),
+    "mlp_down": (8192, 8192, 28672, "normal"),
+    "skinny16": (16, 8192, 8192, "normal"),
+    "skinny64": (64, 8192, 8192, "normal"),
+    "skinny128": (128, 8192, 8192, "normal"),
+    "unaligned": (4095, 6143, 3073, "uniform"),
+}
+# HBM bytes per launch of the 8192^3 kernel measured with rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE (profiles/), scaled by the same counters on a copy kernel of known size.
+MEASURED_TRAFFIC_BYTES = {"square8192": None}
+
+
+def make_inputs(orc, M, N, K, fill, seed=69):
+    if fill == "uniform":
+        return orc.fill_uniform((M, K), seed, 1), orc.fill_uniform((N, K), seed, 2)
+    return orc.fill_normal((M, K), seed, 1, 1.0), orc.fill_normal((N, K), seed, 2, 0.02)
+
+
+def cpu_baseline(orc, A, B, budget_tiles: int) -> dict:
+    """Time the loop-order-faithful oracle on a sample of 64x64 tiles (each tile is the
+    full K deep, exactly the reference's arithmetic for those outputs)."""
+    M, K = A.shape
+    N = B.shape[0]
+    tiles = orc.sample_tiles(M, N, budget_tiles)
+    t0 = time.perf_counter()
+    orc.reference_cpu_gemm(A, B, fast=False, tiles=tiles)
+    dt = time.perf_counter() - t0
+    flops = 0
+    for ti, tj in tiles:
+        flops += 2.0 * min(64, M - ti * 64) * min(64, N - tj * 64) * K
+    total_tiles = -(-M // 64) * -(-N // 64)
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": orc.num_threads(),
+            "kind": "port",
+            "sample": f"{len(tiles)} of {total_tiles} 64x64 output tiles, full K={K}, "
+                      f"reference loop order, {dt:.1f} s; whole problem extrapolates to "
+                      f"{dt * total_tiles / len(tiles):.0f} s"}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="square8192", choices=sorted(WORKLOADS))
+    ap.add_argument("--config", default=None, help="kernel configuration name or index (default: library's choice)")
+    ap.add_argument("--cpu-tiles", type=int, default=1024, help="64x64 tiles in the CPU baseline sample (0 = skip)")
+    ap.add_argument("--check-tiles", type=int, default=64, help="64x64 tiles verified against the oracle (0 = skip)")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
+              "(the GEMM shards by splitting N or M across GPUs with no exchange; see DESIGN.md)",
+              file=sys.stderr)
+        return 2
+    if int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: launched with WORLD_SIZE > 1; one GPU only", file=sys.stderr)
+        return 2
+
+    import h100_gemm_amd as mi          # raises if libmi_gemm.so is not built
+    from oracle import oracle as orc    # checker + CPU baseline only
+
+    M, N, K, fill = WORKLOADS[a.workload]
+    props = mi.device_props()
+    A, B = make_inputs(orc, M, N, K, fill)
+    dA, dB = mi.DeviceBuffer.from_numpy(A), mi.DeviceBuffer.from_numpy(B)
+    dC = mi.DeviceBuffer(M * N * 2)
+    if a.config is None:
+        cfg = mi.select_config(M, N, K)
+    else:
+        cfg = int(a.config) if a.config.lstrip("-").isdigit() else mi.find_config(a.config)
+        if not 0 <= cfg < mi.num_configs():
+            print(f"bench.py: unknown kernel config {a.config!r}", file=sys.stderr)
+            return 2
+    params = mi.GemmParams(M, N, K, dA, dB, dC)
+
+    for _ in range(a.warmup):
+        mi.gpu_gemm(params, config=cfg)
+    mi.synchronize()
+    timer = mi.GPUTimer()                 # HIP events on the launch stream (null stream)
+    t_host0 = time.perf_counter()
+    timer.tick()
+    for _ in range(a.steps):
+        mi.gpu_gemm(params, config=cfg)
+    timer.tick()
+    mi.synchronize()
+    t_host = time.perf_counter() - t_host0
+    ms_total = timer.report_last_ms()
+    ms_per_step = ms_total / a.steps
+
+    # correctness of what was just timed, on a sample of tiles
+    violations = None
+    if a.check_tiles > 0:
+        C = dC.to_numpy((M, N), np.uint16)
+        tiles = orc.sample_tiles(M, N, a.check_tiles)
+        ref = orc.reference_cpu_gemm(A, B, tiles=tiles)
+        rep = orc.check_tolerance(C, ref, K, orc.max_abs(A), orc.max_abs(B), tiles=tiles)
+        violations = rep["violations"]
+
+    flops = 2.0 * M * N * K
+    algo_bytes = 2.0 * (M * K + N * K + M * N)
+    tflops = flops / (ms_per_step * 1e-3) / 1e12
+    gbs = algo_bytes / (ms_per_step * 1e-3) / 1e9
+    ridge = PEAK_BF16_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9)
+    if flops / algo_bytes >= ridge:
+        roof = {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                "frac": tflops / PEAK_BF16_TFLOPS}
+    else:
+        roof = {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "frac": gbs / PEAK_HBM_GBS}
+    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(a.workload)
+    roof["kernel"] = mi.config_name(cfg)
+    roof["avg_launch_us"] = ms_per_step * 1e3
+
+    cpu = cpu_baseline(orc, A, B, a.cpu_tiles) if a.cpu_tiles > 0 else None
+
+    out = {
+        "metric": "bf16 GEMM TFLOP/s at M=N=K=8192 on 1 MI355X; % of bf16 MFMA peak",
+        "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{a.workload}: M={M} N={N} K={K}, A,B {fill} seeded bf16, fp32 accumulate, bf16 out",
+                   "kernel_config": mi.config_name(cfg), "device": props["name"] or props["arch"],
+                   "compute_units": props["compute_units"], "peak_clock_mhz": props["clock_khz"] / 1000},
+        "pct_of_bf16_mfma_peak": 100.0 * tflops / PEAK_BF16_TFLOPS,
+        "achieved_gbs_algorithmic": gbs,
+        "tolerance_violations": violations,
+        "host_wall_ms_per_step": t_host * 1e3 / a.steps,
+        "roofline": roof,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+    return 0 if not violations else 1
+
+
+if __name__ == "__main__":
+    sys.exit(main())
