@@ -65,14 +65,18 @@ struct GemmArgs {
 //   DTL          1: global -> LDS by direct-to-LDS buffer loads (no staging registers, no
 //                ds_write); 0: global -> registers -> ds_write.  The predicated variant
 //                always stages through registers (it has to mask the K tail there).
+//   EPI          1: the aligned kernel transposes its C tile through LDS and writes whole
+//                256-byte row segments (16 bytes per lane); 0: 8-byte stores straight from
+//                the accumulator layout
 //   EDGE         predicated variant: any M, N, K and any alignment
 //   DT           storage type (DT_BF16 / DT_FP16)
-template <int BM_, int BN_, int WM_, int WN_, int SWZ_, int GROUP_, int OCC_, int DTL_, bool EDGE_, int DT_>
+template <int BM_, int BN_, int WM_, int WN_, int SWZ_, int GROUP_, int OCC_, int DTL_, int EPI_, bool EDGE_, int DT_>
 struct TileConfig {
     static constexpr int BM = BM_, BN = BN_, BK = 64;
     static constexpr int WM = WM_, WN = WN_;
     static constexpr int SWZ = SWZ_, GROUP = GROUP_, OCC = OCC_;
     static constexpr bool DTL = DTL_ != 0 && !EDGE_;
+    static constexpr bool EPI = EPI_ != 0 && !EDGE_;
     static constexpr bool EDGE = EDGE_;
     static constexpr int DT = DT_;
     static constexpr int NT = WM * WN * 64;             // threads per workgroup
@@ -547,13 +551,50 @@ gemm_tile_kernel(const GemmArgs p) {
         tr_store = tr_now();
         tr_loop = tr_store - tr_loop;
     }
-    // ---- epilogue: fp32 -> storage type, 8-byte stores into row-major C ----
+    // ---- epilogue: fp32 -> storage type -> row-major C ----
     // acc[i][j][e] of lane l is C[m][n] with m = row of A fragment = l & 31,
     // n = 8*(e/4) + 4*(l>>5) + (e%4) inside the 32x32 tile.
     unsigned char* Cb = (unsigned char*)p.C + (size_t)row0 * p.ldc * 2;
     const uint32_t bytesC = (uint32_t)(rowsA * p.ldc) * 2u;
     const __amdgpu_buffer_rsrc_t rsrcC =
         __builtin_amdgcn_make_buffer_rsrc((void*)Cb, 0, (int)bytesC, 0x00020000);
+    if constexpr (Cfg::EPI) {
+        // Through LDS: each wave lays its TM x TN tile out row-major in its own slice of the
+        // (now idle) stage buffers, 16-byte chunks XOR-swizzled by the row, then reads rows
+        // back 16 bytes per lane so that one store instruction writes whole TN*2-byte row
+        // segments.  Only the first barrier involves the other waves.
+        constexpr int TM = Cfg::TM, TN = Cfg::TN;
+        constexpr int CPR = TN / 8;                 // 16-byte chunks per row of the wave tile
+        constexpr int RPI = 64 / CPR;               // rows one read/store instruction covers
+        static_assert(TM * TN * 2 * Cfg::WM * Cfg::WN <= Cfg::LDS_BYTES, "staging fits the stage buffers");
+        lds_barrier();                              // every wave is done reading the last stage
+        unsigned char* stg = lds + wave * (TM * TN * 2);
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+            const int row = i * 32 + l32;
+#pragma unroll
+            for (int j = 0; j < NI; ++j) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int chunk = (j * 4 + g) ^ (row & (CPR - 1));
+                    u32x2_t w;
+                    w[0] = cvt_store2<DT>(acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1]);
+                    w[1] = cvt_store2<DT>(acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]);
+                    *(u32x2_t*)(stg + row * (TN * 2) + chunk * 16 + hi * 8) = w;
+                }
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // own writes visible to own reads
+        const int rr = lane / CPR, rc = lane % CPR;
+        const uint32_t cbase =
+            (uint32_t)((wm * TM + rr) * p.ldc + col0 + wn * TN + rc * 8) * 2u;
+#pragma unroll
+        for (int r = 0; r < TM / RPI; ++r) {
+            const int row = r * RPI + rr;
+            const u32x4_t v = *(const u32x4_t*)(stg + row * (TN * 2) + ((rc ^ (row & (CPR - 1))) << 4));
+            __builtin_amdgcn_raw_buffer_store_b128(v, rsrcC, cbase + (uint32_t)(r * RPI * p.ldc) * 2u, 0, 0);
+        }
+    } else {
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
         const int m_loc = wm * Cfg::TM + i * 32 + l32;
@@ -587,6 +628,7 @@ gemm_tile_kernel(const GemmArgs p) {
                 }
             }
         }
+    }
     }
     if constexpr (TRACE) {
         if (p.DB != nullptr && tid == 0) {

@@ -10,6 +10,7 @@ template takes (matmul_h100.cu.jinja:9-14) -- re-cast for CDNA4:
     GROUP    tile-order group height (L2 locality of the workgroups sharing an XCD)
     OCC      workgroups per CU the register budget is sized for
     DTL      1: direct-to-LDS global loads in the aligned kernel, 0: register staged
+    EPI      1: C tile transposed through LDS and written 16 bytes per lane, 0: 8-byte stores
 
 The index of a config in ``CONFIGS`` is its ``config`` number in the C ABI.
 """
@@ -18,7 +19,7 @@ from __future__ import annotations
 
 def config_name(c: dict) -> str:
     return (f"t{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_s{c['SWZ']}_g{c['GROUP']}"
-            f"_o{c['OCC']}_d{c['DTL']}")
+            f"_o{c['OCC']}_d{c['DTL']}_e{c['EPI']}")
 
 
 def lds_bytes(c: dict) -> int:
@@ -46,21 +47,21 @@ def is_valid_config(c: dict) -> bool:
     return regs <= 512 // waves_per_simd
 
 
-def _c(BM, BN, WM, WN, SWZ=1, GROUP=8, OCC=1, DTL=0):
-    return dict(BM=BM, BN=BN, WM=WM, WN=WN, SWZ=SWZ, GROUP=GROUP, OCC=OCC, DTL=DTL)
+def _c(BM, BN, WM, WN, SWZ=1, GROUP=8, OCC=1, DTL=0, EPI=0):
+    return dict(BM=BM, BN=BN, WM=WM, WN=WN, SWZ=SWZ, GROUP=GROUP, OCC=OCC, DTL=DTL, EPI=EPI)
 
 
 CONFIGS = [
     _c(256, 256, 2, 2, SWZ=1, GROUP=8),
     _c(256, 256, 2, 2, SWZ=1, GROUP=8, DTL=1),
-    _c(256, 256, 2, 2, SWZ=0, GROUP=8, DTL=1),
+    _c(256, 256, 2, 2, SWZ=1, GROUP=8, DTL=1, EPI=1),
     _c(256, 256, 2, 2, SWZ=1, GROUP=4, DTL=1),
     _c(256, 256, 2, 4, SWZ=1, GROUP=8),
-    _c(256, 256, 2, 4, SWZ=1, GROUP=8, DTL=1),
+    _c(256, 256, 2, 4, SWZ=1, GROUP=8, DTL=1, EPI=1),
     _c(256, 256, 4, 2, SWZ=1, GROUP=8, DTL=1),
     _c(256, 128, 2, 2, SWZ=1, GROUP=8, DTL=1),
     _c(128, 128, 2, 2, SWZ=1, GROUP=8, OCC=2),
-    _c(128, 128, 2, 2, SWZ=1, GROUP=8, OCC=2, DTL=1),
+    _c(128, 128, 2, 2, SWZ=1, GROUP=8, OCC=2, DTL=1, EPI=1),
 ]
 
 assert all(is_valid_config(c) for c in CONFIGS), [config_name(c) for c in CONFIGS if not is_valid_config(c)]

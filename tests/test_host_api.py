@@ -93,8 +93,8 @@ def test_config_table(mi):
                     (16, 8192, 8192), (64, 8192, 8192), (128, 8192, 8192), (4095, 6143, 3073)]:
         assert 0 <= mi.select_config(M, N, K) < n
         assert L.mi_gemm_trace_words(M, N, K) >= 7
-    assert not kc.is_valid_config(dict(BM=256, BN=256, WM=2, WN=2, SWZ=1, GROUP=8, OCC=2, DTL=0))
-    assert not kc.is_valid_config(dict(BM=96, BN=256, WM=2, WN=2, SWZ=1, GROUP=8, OCC=1, DTL=0))
+    assert not kc.is_valid_config(dict(BM=256, BN=256, WM=2, WN=2, SWZ=1, GROUP=8, OCC=2, DTL=0, EPI=0))
+    assert not kc.is_valid_config(dict(BM=96, BN=256, WM=2, WN=2, SWZ=1, GROUP=8, OCC=1, DTL=0, EPI=0))
 
 
 def tile_of_block(pid, nwg, tiles_m, tiles_n, group):
