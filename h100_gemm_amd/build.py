@@ -43,7 +43,7 @@ def render_sources(configs=None) -> list[Path]:
     GEN.mkdir(parents=True, exist_ok=True)
     unit_t = Template((PKG / "template" / "kernel_unit.hip.jinja").read_text())
     table_t = Template((PKG / "template" / "kernel_table.hpp.jinja").read_text())
-    named = [dict(c, name=kc.config_name(c)) for c in configs]
+    named = [dict(c, name=kc.config_name(c), threads=kc.threads(c), lds=kc.lds_bytes(c)) for c in configs]
     units = []
     for c in named:
         p = GEN / f"unit_{c['name']}.hip"
@@ -54,7 +54,9 @@ def render_sources(configs=None) -> list[Path]:
     small = names.index(kc.config_name(kc.DEFAULT_SMALL)) if hasattr(kc, "DEFAULT_SMALL") else len(names) - 1
     _write_if_changed(GEN / "kernel_table.hpp",
                       table_t.render(configs=named, big_index=big, small_index=small,
-                                     big_min_tiles=getattr(kc, "BIG_MIN_TILES", 64)))
+                                     big_min_tiles=getattr(kc, "BIG_MIN_TILES", 64),
+                                     skinny_index=sorted((c["BM"], i) for i, c in enumerate(named)
+                                                         if c["KIND"] == "skinny")))
     # drop units of configs that no longer exist
     keep = {p.name for p in units}
     for old in GEN.glob("unit_*.hip"):
@@ -66,7 +68,8 @@ def render_sources(configs=None) -> list[Path]:
 
 def _stamp(src: Path) -> str:
     h = hashlib.sha1()
-    for dep in [src, CSRC / "gemm_kernel.hpp", CSRC / "gemm_launch.hpp", GEN / "kernel_table.hpp",
+    for dep in [src, CSRC / "gemm_kernel.hpp", CSRC / "gemm_launch.hpp", CSRC / "gemm_ring_kernel.hpp",
+                CSRC / "gemm_skinny_kernel.hpp", GEN / "kernel_table.hpp",
                 PKG.parent / "include" / "mi_gemm.h"]:
         h.update(dep.read_bytes())
     h.update(" ".join(HIPFLAGS).encode())

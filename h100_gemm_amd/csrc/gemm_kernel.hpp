@@ -54,6 +54,8 @@ struct GemmArgs {
     int tiles_m, tiles_n;    // ceil(M/BM), ceil(N/BN)
     int c_vec_ok;            // 1: every C row start is 8-byte aligned (ldc % 4 == 0, base aligned)
     int* DB;                 // optional trace buffer (may be null)
+    float* ws;               // split-K workspace (decode kernels only)
+    int splits, k_per_split; // split-K geometry (decode kernels only)
 };
 
 // Compile-time description of one kernel variant -- the knobs the tuner sweeps.
@@ -230,12 +232,18 @@ gemm_tile_kernel(const GemmArgs p) {
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
     auto gload_a = [&](int kt) __attribute__((always_inline)) {
+#ifdef MI_EXP_NO_GLOAD
+        if (K > 128) return;
+#endif
         const uint32_t kb = (uint32_t)kt * (BK * 2);
 #pragma unroll
         for (int j = 0; j < LA; ++j)
             ga[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrcA, voffA + kb + j * passA, 0, 0);
     };
     auto gload_b = [&](int kt) __attribute__((always_inline)) {
+#ifdef MI_EXP_NO_GLOAD
+        if (K > 128) return;
+#endif
         const uint32_t kb = (uint32_t)kt * (BK * 2);
 #pragma unroll
         for (int j = 0; j < LB; ++j)
@@ -286,13 +294,21 @@ gemm_tile_kernel(const GemmArgs p) {
     };
     auto lds_store_a = [&](int stage) __attribute__((always_inline)) {
 #pragma unroll
-        for (int j = 0; j < LA; ++j)
+        for (int j = 0; j < LA; ++j) {
+#ifdef MI_EXP_NO_LDS_STORE
+            if (K > 128) { asm volatile("" :: "v"(ga[j])); continue; }
+#endif
             *(u32x4_t*)(lds + stage * A_STAGE + wr_off + j * (RPP * 128)) = ga[j];
+        }
     };
     auto lds_store_b = [&](int stage) __attribute__((always_inline)) {
 #pragma unroll
-        for (int j = 0; j < LB; ++j)
+        for (int j = 0; j < LB; ++j) {
+#ifdef MI_EXP_NO_LDS_STORE
+            if (K > 128) { asm volatile("" :: "v"(gb[j])); continue; }
+#endif
             *(u32x4_t*)(lds + 2 * A_STAGE + stage * B_STAGE + wr_off + j * (RPP * 128)) = gb[j];
+        }
     };
     auto read_frags = [&](int stage, int ks, int buf) __attribute__((always_inline)) {
 #pragma unroll

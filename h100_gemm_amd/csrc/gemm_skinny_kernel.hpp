@@ -1,0 +1,230 @@
+// gemm_skinny_kernel.hpp -- gfx950 GEMM kernel for decode-shaped problems (M <= 128):
+//
+//   C[M,N] = A[M,K] . B[N,K]^T     M small, B (the weights) streamed once from HBM
+//
+// These shapes are bound by the HBM read of B, not by MFMA, so the kernel is organised
+// around keeping bytes of B in flight on every CU:
+//   * a workgroup owns BN = 128 rows of B and a slice of K (split-K over blockIdx.y), which
+//     gives >= 256 workgroups for N = 8192 while each still amortises its A reads over
+//     128 columns;
+//   * B and A slabs (64 k deep, 128-byte rows, XOR-swizzled) go global -> LDS through
+//     direct-to-LDS buffer loads into a ring of NS stages; NS-1 slabs are always in flight;
+//   * one s_barrier per slab; waits are `vmcnt((NS-2)*L)`, never on the youngest loads;
+//   * each of the 4 waves multiplies all BM rows with its own 32 columns
+//     (v_mfma_f32_32x32x16, operands swapped so a lane holds 4 consecutive n);
+//   * with split-K the fp32 partial tiles go to a workspace and splitk_reduce_kernel adds
+//     them in a fixed order (so results are reproducible) and rounds once to the storage
+//     type; without split-K the tile is rounded and stored directly.
+// The reference has no counterpart: its kernels assert M % 128 == 0 (matmul_utils.cuh:362,
+// 386-387).  Rows of A past M are never fetched (the buffer descriptor ends at row M-1 and
+// out-of-range loads return zero).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "gemm_kernel.hpp"
+
+namespace mi {
+
+struct SkinnyArgs {
+    const void* A;
+    const void* B;
+    void* C;          // storage-type output (used when splits == 1)
+    float* ws;        // [splits][M][N] fp32 partials (used when splits > 1)
+    int M, N, K;
+    int lda, ldb, ldc;
+    int k_per_split;  // multiple of 64
+    int splits;
+};
+
+template <int BM_, int BN_, int NS_, int DT_>
+struct SkinnyConfig {
+    static constexpr int BM = BM_, BN = BN_, NS = NS_, DT = DT_;
+    static constexpr int NT = 256, NW = 4;
+    static constexpr int MI = BM / 32;                       // 32-row MFMA blocks
+    static constexpr int TN = BN / NW;                       // columns per wave
+    static constexpr int NI = TN / 32;
+    static constexpr int ROWS = BM + BN;                     // rows of one stage: A then B
+    static constexpr int STAGE = ROWS * 128;
+    static constexpr int L = ROWS / 8 / NW;                  // load instructions per wave per slab
+    static constexpr int LDS_BYTES = NS * STAGE;
+    static_assert(BM % 32 == 0 && TN % 32 == 0, "MFMA blocks are 32x32");
+    static_assert((ROWS / 8) % NW == 0, "load instructions divide over the waves");
+    static_assert(NS >= 2 && (NS - 1) * L <= 63, "vmcnt is a 6-bit counter");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
+};
+
+template <class Cfg>
+__global__ void __launch_bounds__(256) gemm_skinny_kernel(const SkinnyArgs p) {
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::NS, DT = Cfg::DT;
+    constexpr int MI = Cfg::MI, NI = Cfg::NI, TN = Cfg::TN, L = Cfg::L, STAGE = Cfg::STAGE;
+
+    __shared__ __attribute__((aligned(128))) unsigned char lds[Cfg::LDS_BYTES];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int col0 = blockIdx.x * BN;
+    const int split = blockIdx.y;
+    const int M = p.M, N = p.N, K = p.K;
+    const int k0 = split * p.k_per_split;
+    const int kend = (k0 + p.k_per_split) < K ? (k0 + p.k_per_split) : K;
+    const int KT = (kend - k0) / 64;                         // slabs of this split (>= 1)
+
+    const int rowsA = M < BM ? M : BM;
+    const int rowsB = (N - col0) < BN ? (N - col0) : BN;
+    const unsigned char* Ab = (const unsigned char*)p.A + (size_t)k0 * 2;
+    const unsigned char* Bb = (const unsigned char*)p.B + ((size_t)col0 * p.ldb + k0) * 2;
+    // descriptors end at the last element this split needs of the last valid row
+    const uint32_t bytesA = (uint32_t)((rowsA - 1) * p.lda + (kend - k0)) * 2u;
+    const uint32_t bytesB = (uint32_t)((rowsB - 1) * p.ldb + (kend - k0)) * 2u;
+    const __amdgpu_buffer_rsrc_t rsrcA = __builtin_amdgcn_make_buffer_rsrc((void*)Ab, 0, (int)bytesA, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrcB = __builtin_amdgcn_make_buffer_rsrc((void*)Bb, 0, (int)bytesB, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrcNone = __builtin_amdgcn_make_buffer_rsrc((void*)Ab, 0, 0, 0x00020000);
+
+    // One load instruction fills 8 consecutive 128-byte rows of a stage: lane l lands on
+    // chunk position l & 7 of row l >> 3 and therefore fetches logical chunk
+    // (l & 7) ^ swz(row), swz(row) = (row >> 1) & 7.  Instruction q (0 .. ROWS/8-1) of a slab
+    // covers stage rows 8q .. 8q+7; rows below BM belong to A, the rest to B; wave w issues
+    // q = w, w + 4, ...
+    const int lr = lane >> 3, lc = lane & 7;
+    auto swz = [](int row) __attribute__((always_inline)) { return (row >> 1) & 7; };
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
+    auto dma = [&](const __amdgpu_buffer_rsrc_t& rsrc, uint32_t voff, uint32_t dst) __attribute__((always_inline)) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                     :: "s"(dst), "v"(voff), "s"(rsrc) : "memory");
+    };
+    auto dma_slab = [&](int t, int s) __attribute__((always_inline)) {
+        const bool live = t < KT;
+        const uint32_t kb = (uint32_t)t * 128u;
+#pragma unroll
+        for (int i = 0; i < L; ++i) {
+            const int q = wave + i * 4;                      // wave-uniform
+            const int row = q * 8 + lr;                      // stage row of this lane
+            const int chunk = lc ^ swz(row);
+            const uint32_t dst = lds_base + (uint32_t)(s * STAGE + q * 1024);
+            if (q * 8 < BM) {
+                dma(live ? rsrcA : rsrcNone, (uint32_t)(row * p.lda + chunk * 8) * 2u + kb, dst);
+            } else {
+                dma(live ? rsrcB : rsrcNone, (uint32_t)((row - BM) * p.ldb + chunk * 8) * 2u + kb, dst);
+            }
+        }
+    };
+
+    // fragment reads: lane holds row (lane & 31), k chunk 2*ks + (lane >> 5)
+    const int l32 = lane & 31, hi = lane >> 5;
+    int rd_off[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) rd_off[ks] = l32 * 128 + ((((ks << 1) | hi) ^ swz(l32)) << 4);
+    const int b_wave = (BM + wave * TN) * 128;
+
+    f32x16_t acc[MI][NI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+    // ---- prologue: slabs 0 .. NS-2 in flight ----
+#pragma unroll
+    for (int t = 0; t < NS - 1; ++t) dma_slab(t, t);
+
+    int s = 0;
+    for (int t = 0; t < KT; ++t) {
+        // slab t has landed for every wave, and every wave is done with slab t-1
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" :: "n"((NS - 2) * L) : "memory");
+        // refill the stage that slab t-1 occupied
+        dma_slab(t + NS - 1, s == 0 ? NS - 1 : s - 1);
+        const unsigned char* st = lds + s * STAGE;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            u32x4_t fa[MI], fb[NI];
+#pragma unroll
+            for (int i = 0; i < MI; ++i) fa[i] = *(const u32x4_t*)(st + i * 4096 + rd_off[ks]);
+#pragma unroll
+            for (int j = 0; j < NI; ++j) fb[j] = *(const u32x4_t*)(st + b_wave + j * 4096 + rd_off[ks]);
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int j = 0; j < NI; ++j) acc[i][j] = mfma_32x32x16<DT>(fb[j], fa[i], acc[i][j]);
+        }
+        s = s + 1 == NS ? 0 : s + 1;
+    }
+    // loads requested past this split's K range are still heading for the ring
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    // ---- epilogue: lane holds C[m][n..n+3], m = i*32 + (lane & 31), n = 8g + 4*(lane>>5) ----
+    if (p.splits == 1) {
+        unsigned char* Cb = (unsigned char*)p.C;
+        const __amdgpu_buffer_rsrc_t rsrcC =
+            __builtin_amdgcn_make_buffer_rsrc((void*)Cb, 0, (int)((uint32_t)(M * p.ldc) * 2u), 0x00020000);
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+            const int m = i * 32 + l32;
+#pragma unroll
+            for (int j = 0; j < NI; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int n = col0 + wave * TN + j * 32 + g * 8 + hi * 4;
+                    if (m < M && n < N) {           // N % 4 == 0 is a launch precondition
+                        u32x2_t w;
+                        w[0] = cvt_store2<DT>(acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1]);
+                        w[1] = cvt_store2<DT>(acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]);
+                        __builtin_amdgcn_raw_buffer_store_b64(w, rsrcC, (uint32_t)(m * p.ldc + n) * 2u, 0, 0);
+                    }
+                }
+        }
+    } else {
+        float* P = p.ws + (size_t)split * M * N;
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+            const int m = i * 32 + l32;
+#pragma unroll
+            for (int j = 0; j < NI; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int n = col0 + wave * TN + j * 32 + g * 8 + hi * 4;
+                    if (m < M && n < N) {
+                        float4 v = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2],
+                                    acc[i][j][g * 4 + 3]};
+                        *(float4*)(P + (size_t)m * N + n) = v;
+                    }
+                }
+        }
+    }
+}
+
+// C[m][n] = round(sum over splits, in split order, of ws[s][m][n]); 4 elements per thread.
+template <int DT>
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restrict__ ws, void* C, int M,
+                                                            int N, int ldc, int splits) {
+    const size_t idx = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    const size_t total = (size_t)M * N;
+    if (idx >= total) return;
+    float4 a = *(const float4*)(ws + idx);
+    for (int s = 1; s < splits; ++s) {
+        const float4 b = *(const float4*)(ws + (size_t)s * total + idx);
+        a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+    }
+    const size_t m = idx / N, n = idx % N;
+    u32x2_t w;
+    w[0] = cvt_store2<DT>(a.x, a.y);
+    w[1] = cvt_store2<DT>(a.z, a.w);
+    *(u32x2_t*)((unsigned char*)C + (m * ldc + n) * 2) = w;
+}
+
+template <class Cfg>
+hipError_t launch_skinny_kernel(const SkinnyArgs& a, hipStream_t stream) {
+    dim3 grid((a.N + Cfg::BN - 1) / Cfg::BN, a.splits);
+    hipLaunchKernelGGL((gemm_skinny_kernel<Cfg>), grid, dim3(256), 0, stream, a);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || a.splits == 1) return e;
+    const size_t quads = ((size_t)a.M * a.N + 3) / 4;
+    hipLaunchKernelGGL((splitk_reduce_kernel<Cfg::DT>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0,
+                       stream, a.ws, a.C, a.M, a.N, a.ldc, a.splits);
+    return hipGetLastError();
+}
+
+}  // namespace mi

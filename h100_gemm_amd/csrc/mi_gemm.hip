@@ -11,7 +11,9 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 #include "../../include/mi_gemm.h"
 #include "gemm_kernel.hpp"
@@ -43,6 +45,63 @@ int fail(int code, const char* fmt, ...) {
     } while (0)
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+// Preconditions of the decode (split-K streaming) kernels: whole 16-byte chunks and whole
+// 64-deep K slabs, 8-byte aligned C rows.
+bool shape_is_streamable(int M, int N, int K, const void* A, const void* B, const void* C) {
+    return M <= 128 && N % 4 == 0 && K % 64 == 0 && aligned16(A) && aligned16(B) &&
+           (((uintptr_t)C & 7u) == 0);
+}
+
+// Split-K geometry for a decode launch: aim at two workgroups per CU, keep at least four
+// K slabs per split.  MI_GEMM_SPLITK=<n> overrides (tuning aid).
+int choose_splits(int tiles_n, int K, int cus) {
+    static const int env = [] { const char* s = getenv("MI_GEMM_SPLITK"); return s ? atoi(s) : 0; }();
+    const int slabs = K / 64;
+    int splits = env > 0 ? env : (2 * cus + tiles_n - 1) / tiles_n;
+    if (splits > slabs / 4) splits = slabs / 4;
+    if (splits < 1) splits = 1;
+    if (splits > 64) splits = 64;
+    return splits;
+}
+
+// fp32 partial-sum workspace of the split-K kernels: one buffer per process, grown on
+// demand.  Launches that use it are ordered on their stream; callers that run split-K
+// launches on several streams at once must serialise them.
+std::mutex g_ws_mutex;
+float* g_ws = nullptr;
+size_t g_ws_bytes = 0;
+int g_cus = 0;
+
+hipError_t ensure_workspace(size_t bytes, float** out) {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    if (bytes > g_ws_bytes) {
+        if (g_ws) {
+            hipError_t e = hipFree(g_ws);      // waits for work that may still use it
+            g_ws = nullptr;
+            g_ws_bytes = 0;
+            if (e != hipSuccess) return e;
+        }
+        const size_t want = bytes < (size_t)(32u << 20) ? (size_t)(32u << 20) : bytes;
+        hipError_t e = hipMalloc((void**)&g_ws, want);
+        if (e != hipSuccess) return e;
+        g_ws_bytes = want;
+    }
+    *out = g_ws;
+    return hipSuccess;
+}
+
+int compute_units() {
+    if (g_cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            g_cus = n;
+        else
+            g_cus = 256;
+    }
+    return g_cus;
+}
 
 // The aligned kernels assume full tiles, K a multiple of two K steps, 16-byte aligned
 // rows of A and B and 8-byte aligned rows of C; everything else takes the predicated twin.
@@ -99,19 +158,26 @@ int mi_gemm_config_supports(int config, int dtype, int M, int N, int K) {
     if (config < 0 || config >= mi::kNumKernels) return 0;
     if (dtype != MI_DTYPE_BF16 && dtype != MI_DTYPE_FP16) return 0;
     if (M <= 0 || N <= 0 || K <= 0) return 0;
-    return mi::kKernels[config].launch[dtype][1] != nullptr;
+    const mi::KernelEntry& e = mi::kKernels[config];
+    if (e.kind == mi::KIND_SKINNY) return M <= e.BM && N % 4 == 0 && K % 64 == 0;
+    return e.launch[dtype][1] != nullptr;
 }
 
 int mi_gemm_config_grid(int config, int M, int N, int K) {
     if (config < 0 || config >= mi::kNumKernels || M <= 0 || N <= 0 || K <= 0) return 0;
     const mi::KernelEntry& e = mi::kKernels[config];
+    if (e.kind == mi::KIND_SKINNY) {
+        if (M > e.BM || K % 64 != 0) return 0;
+        const int tiles_n = (N + e.BN - 1) / e.BN;
+        return tiles_n * choose_splits(tiles_n, K, compute_units());
+    }
     return ((M + e.BM - 1) / e.BM) * ((N + e.BN - 1) / e.BN);
 }
 
 int mi_gemm_select_config(int dtype, int M, int N, int K) {
     (void)dtype;
-    (void)K;
-    return mi::select_kernel(M, N, K);
+    // pointer alignment is unknown here: assume the usual 256-byte aligned allocations
+    return mi::select_kernel(M, N, K, M <= 128 && N % 4 == 0 && K % 64 == 0);
 }
 
 size_t mi_gemm_trace_words(int M, int N, int K) {
@@ -128,7 +194,8 @@ int mi_gemm_ex(int config, int dtype, int M, int N, int K, const void* A, const 
                void* C, int* DB, void* stream) {
     int rc = check_args(config, dtype, M, N, K, A, B, C);
     if (rc != MI_OK) return rc;
-    if (config == MI_CONFIG_AUTO) config = mi::select_kernel(M, N, K);
+    const bool streamable = shape_is_streamable(M, N, K, A, B, C);
+    if (config == MI_CONFIG_AUTO) config = mi::select_kernel(M, N, K, streamable);
     const mi::KernelEntry& e = mi::kKernels[config];
 
     mi::GemmArgs args;
@@ -145,6 +212,30 @@ int mi_gemm_ex(int config, int dtype, int M, int N, int K, const void* A, const 
     args.tiles_n = (N + e.BN - 1) / e.BN;
     args.c_vec_ok = (N % 4 == 0) && (((uintptr_t)C & 7u) == 0);
     args.DB = DB;
+    args.ws = nullptr;
+    args.splits = 1;
+    args.k_per_split = K;
+
+    if (e.kind == mi::KIND_SKINNY) {
+        if (!streamable || M > e.BM)
+            return fail(MI_ERR_UNSUPPORTED,
+                        "config %s needs M <= %d, N %% 4 == 0, K %% 64 == 0 and 16-byte aligned operands",
+                        e.name, e.BM);
+        const int tiles_n = (N + e.BN - 1) / e.BN;
+        args.splits = choose_splits(tiles_n, K, compute_units());
+        const int slabs = K / 64;
+        args.k_per_split = ((slabs + args.splits - 1) / args.splits) * 64;
+        args.splits = (K + args.k_per_split - 1) / args.k_per_split;   // no empty split
+        if (args.splits > 1) {
+            hipError_t we = ensure_workspace((size_t)args.splits * M * N * sizeof(float), &args.ws);
+            if (we != hipSuccess)
+                return fail(MI_ERR_HIP, "split-K workspace allocation failed: %s", hipGetErrorString(we));
+        }
+        hipError_t err = e.launch[dtype][0](args, (hipStream_t)stream);
+        if (err != hipSuccess)
+            return fail(MI_ERR_HIP, "launch of %s failed: %s", e.name, hipGetErrorString(err));
+        return MI_OK;
+    }
 
     const bool edge = !shape_is_aligned(e, M, N, K, A, B, C);
     mi::LaunchFn fn = e.launch[dtype][edge ? 1 : 0];

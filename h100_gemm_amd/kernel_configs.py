@@ -10,6 +10,9 @@ template takes (matmul_h100.cu.jinja:9-14) -- re-cast for CDNA4:
     GROUP    tile-order group height (L2 locality of the workgroups sharing an XCD)
     OCC      workgroups per CU the register budget is sized for
     DTL      1: direct-to-LDS global loads in the aligned kernel, 0: register staged
+    KIND     "tile" (two-stage kernel above), "ring" (NS-deep LDS ring, K step 32, aligned
+             shapes; ragged shapes take the predicated tile kernel of the same tile), or
+             "skinny" (split-K streaming kernel for M <= BM, decode shapes)
     EPI      1: C tile transposed through LDS and written 16 bytes per lane, 0: 8-byte stores
 
 The index of a config in ``CONFIGS`` is its ``config`` number in the C ABI.
@@ -18,50 +21,89 @@ from __future__ import annotations
 
 
 def config_name(c: dict) -> str:
+    if c["KIND"] == "ring":
+        return f"r{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_n{c['NS']}_g{c['GROUP']}"
+    if c["KIND"] == "skinny":
+        return f"k{c['BM']}x{c['BN']}_n{c['NS']}"
     return (f"t{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_s{c['SWZ']}_g{c['GROUP']}"
             f"_o{c['OCC']}_d{c['DTL']}_e{c['EPI']}")
 
 
+def threads(c: dict) -> int:
+    return 256 if c["KIND"] == "skinny" else c["WM"] * c["WN"] * 64
+
+
 def lds_bytes(c: dict) -> int:
+    if c["KIND"] == "ring":
+        return c["NS"] * (c["BM"] + c["BN"]) * 64
+    if c["KIND"] == "skinny":
+        return c["NS"] * (c["BM"] + c["BN"]) * 128
     return 2 * (c["BM"] + c["BN"]) * 128
 
 
 def is_valid_config(c: dict) -> bool:
-    """Static rules of gemm_kernel.hpp (mirrored as static_asserts there)."""
+    """Static rules of the kernels (mirrored as static_asserts in csrc/)."""
+    if c["KIND"] == "skinny":
+        return (c["BM"] % 32 == 0 and c["BN"] % 128 == 0 and c["NS"] >= 2
+                and ((c["BM"] + c["BN"]) // 8) % 4 == 0
+                and (c["NS"] - 1) * ((c["BM"] + c["BN"]) // 32) <= 63
+                and lds_bytes(c) <= 160 * 1024)
     nt = c["WM"] * c["WN"] * 64
     if nt > 1024 or nt < 64:
         return False
     if c["BM"] % (32 * c["WM"]) or c["BN"] % (32 * c["WN"]):
         return False
-    if (c["BM"] * 8) % nt or (c["BN"] * 8) % nt or (nt // 8) % 16:
-        return False
-    if lds_bytes(c) * c["OCC"] > 160 * 1024:
-        return False
     mi, ni = c["BM"] // c["WM"] // 32, c["BN"] // c["WN"] // 32
     nmma = mi * ni
+    occ = c.get("OCC", 1)
+    if lds_bytes(c) * occ > 160 * 1024:
+        return False
+    waves_per_simd = max(nt // 256, 1) * occ
+    if c["KIND"] == "ring":
+        rpp = (nt // 64) * 16
+        if c["BM"] % rpp or c["BN"] % rpp or c["NS"] != 4:
+            return False
+        l = c["BM"] // rpp + c["BN"] // rpp
+        if l % 2 or l // 2 > nmma - (mi + ni) or (c["NS"] - 2) * l > 63:
+            return False
+        if c["BM"] * c["BN"] * 2 > lds_bytes(c):
+            return False
+        return nmma * 16 + 2 * (mi + ni) * 4 + 40 <= 512 // waves_per_simd
+    if (c["BM"] * 8) % nt or (c["BN"] * 8) % nt or (nt // 8) % 16:
+        return False
     if mi + ni > nmma or c["BM"] * 8 // nt > nmma or c["BN"] * 8 // nt > nmma:
         return False
     # accumulators (16 regs per 32x32 tile) + fragments + staging must fit 512 / waves-per-SIMD
-    waves_per_simd = max(nt // 256, 1) * c["OCC"]
     regs = nmma * 16 + 2 * (mi + ni) * 4 + (c["BM"] + c["BN"]) * 8 // nt * 4 + 40
     return regs <= 512 // waves_per_simd
 
 
 def _c(BM, BN, WM, WN, SWZ=1, GROUP=8, OCC=1, DTL=0, EPI=0):
-    return dict(BM=BM, BN=BN, WM=WM, WN=WN, SWZ=SWZ, GROUP=GROUP, OCC=OCC, DTL=DTL, EPI=EPI)
+    return dict(KIND="tile", BM=BM, BN=BN, WM=WM, WN=WN, SWZ=SWZ, GROUP=GROUP, OCC=OCC, DTL=DTL, EPI=EPI)
+
+
+def _r(BM, BN, WM, WN, NS=4, GROUP=8):
+    return dict(KIND="ring", BM=BM, BN=BN, WM=WM, WN=WN, NS=NS, GROUP=GROUP)
+
+
+def _k(BM, BN=128, NS=4):
+    return dict(KIND="skinny", BM=BM, BN=BN, NS=NS)
 
 
 CONFIGS = [
     _c(256, 256, 2, 2, SWZ=1, GROUP=8),
     _c(256, 256, 2, 2, SWZ=1, GROUP=8, DTL=1),
     _c(256, 256, 2, 2, SWZ=1, GROUP=8, DTL=1, EPI=1),
-    _c(256, 256, 2, 2, SWZ=1, GROUP=4, DTL=1),
-    _c(256, 256, 2, 4, SWZ=1, GROUP=8),
+    _c(256, 256, 2, 2, SWZ=1, GROUP=4, DTL=1, EPI=1),
     _c(256, 256, 2, 4, SWZ=1, GROUP=8, DTL=1, EPI=1),
-    _c(256, 256, 4, 2, SWZ=1, GROUP=8, DTL=1),
-    _c(256, 128, 2, 2, SWZ=1, GROUP=8, DTL=1),
-    _c(128, 128, 2, 2, SWZ=1, GROUP=8, OCC=2),
+    _c(256, 128, 2, 2, SWZ=1, GROUP=8, DTL=1, EPI=1),
+    _c(128, 256, 2, 2, SWZ=1, GROUP=8, DTL=1, EPI=1),
     _c(128, 128, 2, 2, SWZ=1, GROUP=8, OCC=2, DTL=1, EPI=1),
+    _r(256, 256, 2, 2),
+    _r(256, 256, 2, 4),
+    _k(32),
+    _k(64),
+    _k(128),
 ]
 
 assert all(is_valid_config(c) for c in CONFIGS), [config_name(c) for c in CONFIGS if not is_valid_config(c)]
@@ -69,6 +111,6 @@ assert len({config_name(c) for c in CONFIGS}) == len(CONFIGS)
 
 # What MI_CONFIG_AUTO resolves to: the big tile when there are enough 256x256 tiles to
 # occupy the chip, the small one otherwise.
-DEFAULT_BIG = CONFIGS[0]
-DEFAULT_SMALL = CONFIGS[8]
+DEFAULT_BIG = CONFIGS[2]
+DEFAULT_SMALL = CONFIGS[7]
 BIG_MIN_TILES = 64

@@ -89,9 +89,9 @@ def test_c5_unaligned_full(mi, orc):
 
 # ------------------------------------------------------ every kernel configuration ----
 
-def all_configs():
+def all_configs(kinds=("tile", "ring")):
     from h100_gemm_amd import kernel_configs as kc
-    return list(range(len(kc.CONFIGS)))
+    return [i for i, c in enumerate(kc.CONFIGS) if c["KIND"] in kinds]
 
 
 @pytest.mark.parametrize("config", all_configs())
@@ -105,6 +105,40 @@ def test_every_config_bit_exact_on_integer_fill(mi, orc, config):
 def test_every_config_uniform_within_tolerance(mi, orc, config):
     for M, N, K in [(1024, 768, 256), (255, 511, 129)]:
         check(mi, orc, M, N, K, "uniform", config=config)
+
+
+# ------------------------------------------------ decode (split-K streaming) kernels ----
+
+@pytest.mark.parametrize("config", all_configs(("skinny",)))
+def test_decode_kernels(mi, orc, config):
+    from h100_gemm_amd import kernel_configs as kc
+    bm = kc.CONFIGS[config]["BM"]
+    for M in sorted({1, bm // 2 + 1, bm - 1, bm}):
+        for N, K in [(128, 64), (8192, 4096), (1028, 8192), (260, 192), (4, 1024)]:
+            check(mi, orc, M, N, K, "int", config=config, exact=True)     # split-K sums of exact ints
+    check(mi, orc, bm, 8192, 8192, "normal", config=config)
+    check(mi, orc, bm, 2048, 512, "uniform", config=config, dtype=orc.FP16)
+    # shapes the kernel cannot run are refused, not mis-computed
+    A, B = make_inputs(orc, bm + 1, 256, 128, "int")
+    d = Dev(mi, A, B, bm + 1, 256)
+    with pytest.raises(mi.MiGemmError) as ei:
+        d.run(128, config=config)
+    assert ei.value.code == mi._lib.MI_ERR_UNSUPPORTED
+    A, B = make_inputs(orc, 8, 256, 100, "int")
+    with pytest.raises(mi.MiGemmError):
+        Dev(mi, A, B, 8, 256).run(100, config=config)
+
+
+def test_decode_dispatch_and_determinism(mi, orc):
+    # automatic choice: decode kernel when its preconditions hold, the predicated tile kernel
+    # otherwise -- same answers either way
+    for M, N, K in [(16, 8192, 8192), (100, 4100, 2112), (128, 8190, 1024), (5, 256, 8200), (128, 8192, 8192)]:
+        check(mi, orc, M, N, K, "int", exact=True)
+    A, B = make_inputs(orc, 64, 8192, 8192, "normal")
+    d = Dev(mi, A, B, 64, 8192)
+    C0 = d.run(8192)
+    for _ in range(3):
+        assert (d.run(8192) == C0).all()          # fixed split order: bit-reproducible
 
 
 # --------------------------------------------------------------------- edge cases ----

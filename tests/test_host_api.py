@@ -84,17 +84,32 @@ def test_config_table(mi):
     for i, c in enumerate(kc.CONFIGS):
         assert L.mi_gemm_config_lds_bytes(i) == kc.lds_bytes(c) <= 160 * 1024
         assert kc.is_valid_config(c)
-        tiles = -(-1000 // c["BM"]) * -(-777 // c["BN"])
-        assert mi.config_grid(i, 1000, 777, 64) == tiles
-        assert L.mi_gemm_config_supports(i, 0, 4095, 6143, 3073) == 1
+        if c["KIND"] == "skinny":
+            # decode kernels: M <= BM, whole 64-deep K slabs, N a multiple of 4; no ragged twin
+            assert L.mi_gemm_config_supports(i, 0, c["BM"], 8192, 8192) == 1
+            assert L.mi_gemm_config_supports(i, 0, c["BM"] + 1, 8192, 8192) == 0
+            assert L.mi_gemm_config_supports(i, 0, 16, 8192, 8200) == 0
+            assert L.mi_gemm_config_supports(i, 0, 16, 8190, 8192) == 0
+            assert mi.config_grid(i, 16, 8192, 8192) >= 64
+            assert mi.config_grid(i, c["BM"] + 1, 8192, 8192) == 0
+        else:
+            tiles = -(-1000 // c["BM"]) * -(-777 // c["BN"])
+            assert mi.config_grid(i, 1000, 777, 64) == tiles
+            assert L.mi_gemm_config_supports(i, 0, 4095, 6143, 3073) == 1
     assert mi.config_grid(0, 0, 8, 8) == 0
     # the automatic choice is a valid index for every benchmark shape
     for M, N, K in [(512, 512, 512), (8192, 8192, 8192), (8192, 28672, 8192), (8192, 8192, 28672),
                     (16, 8192, 8192), (64, 8192, 8192), (128, 8192, 8192), (4095, 6143, 3073)]:
         assert 0 <= mi.select_config(M, N, K) < n
         assert L.mi_gemm_trace_words(M, N, K) >= 7
-    assert not kc.is_valid_config(dict(BM=256, BN=256, WM=2, WN=2, SWZ=1, GROUP=8, OCC=2, DTL=0, EPI=0))
-    assert not kc.is_valid_config(dict(BM=96, BN=256, WM=2, WN=2, SWZ=1, GROUP=8, OCC=1, DTL=0, EPI=0))
+    kinds = {kc.CONFIGS[mi.select_config(M, 8192, 8192)]["KIND"] for M in (16, 64, 128)}
+    assert kinds == {"skinny"}
+    assert kc.CONFIGS[mi.select_config(16, 8192, 8200)]["KIND"] != "skinny"     # K % 64 != 0
+    assert kc.CONFIGS[mi.select_config(8192, 8192, 8192)]["KIND"] in ("tile", "ring")
+    assert not kc.is_valid_config(dict(KIND="tile", BM=256, BN=256, WM=2, WN=2, SWZ=1, GROUP=8, OCC=2, DTL=0, EPI=0))
+    assert not kc.is_valid_config(dict(KIND="tile", BM=96, BN=256, WM=2, WN=2, SWZ=1, GROUP=8, OCC=1, DTL=0, EPI=0))
+    assert not kc.is_valid_config(dict(KIND="ring", BM=256, BN=256, WM=2, WN=2, NS=5, GROUP=8))
+    assert not kc.is_valid_config(dict(KIND="skinny", BM=48, BN=128, NS=4))
 
 
 def tile_of_block(pid, nwg, tiles_m, tiles_n, group):
