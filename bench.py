@@ -81,8 +81,11 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="square8192", choices=sorted(WORKLOADS))
     ap.add_argument("--config", default=None, help="kernel configuration name or index (default: library's choice)")
-    ap.add_argument("--cpu-tiles", type=int, default=1024, help="64x64 tiles in the CPU baseline sample (0 = skip)")
+    ap.add_argument("--cpu-tiles", type=int, default=2048, help="64x64 tiles in the CPU baseline sample (0 = skip)")
     ap.add_argument("--check-tiles", type=int, default=64, help="64x64 tiles verified against the oracle (0 = skip)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain device-to-device copy of 256 MiB (a kernel of known HBM "
+                         "traffic, for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
@@ -110,6 +113,14 @@ def main() -> int:
             return 2
     params = mi.GemmParams(M, N, K, dA, dB, dC)
 
+    if a.calibrate_copy:
+        nbytes = 256 << 20
+        src, dst = mi.DeviceBuffer(nbytes), mi.DeviceBuffer(nbytes)
+        src.fill_bytes(1)
+        mi._lib.check(mi._lib.load().mi_memcpy_d2d(dst.ptr, src.ptr, nbytes))
+        mi.synchronize()
+        src.free()
+        dst.free()
     for _ in range(a.warmup):
         mi.gpu_gemm(params, config=cfg)
     mi.synchronize()

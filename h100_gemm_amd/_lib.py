@@ -52,6 +52,7 @@ SYMBOLS = {
     "mi_free": (C.c_int, [C.c_void_p]),
     "mi_memcpy_h2d": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "mi_memcpy_d2h": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
+    "mi_memcpy_d2d": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "mi_memset": (C.c_int, [C.c_void_p, C.c_int, C.c_size_t]),
     "mi_device_sync": (C.c_int, []),
     "mi_stream_sync": (C.c_int, [C.c_void_p]),

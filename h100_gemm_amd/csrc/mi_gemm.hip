@@ -282,6 +282,10 @@ int mi_memcpy_d2h(void* dst, const void* src, size_t bytes) {
     MI_HIP(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
     return MI_OK;
 }
+int mi_memcpy_d2d(void* dst, const void* src, size_t bytes) {
+    MI_HIP(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToDevice));
+    return MI_OK;
+}
 int mi_memset(void* dst, int value, size_t bytes) {
     MI_HIP(hipMemset(dst, value, bytes));
     return MI_OK;

@@ -1,0 +1,314 @@
+"""Grid-search tuner for the MI355X GEMM kernels.
+
+The counterpart of the reference's ``gemm_tuner.py`` (gemm_tuner.py:11-181), with the same
+class, methods, control flow, failure handling and output files, retargeted from Hopper to
+CDNA4:
+
+* the search space is MFMA macro tile, wave grid, pipeline kind/depth, LDS swizzle, tile-order
+  group, load path and epilogue instead of cluster shape / block / TMA stages
+  (gemm_tuner.py:17-24);
+* a configuration is rendered from ``template/matmul_mi355x.hip.jinja``, compiled with
+  ``hipcc --offload-arch=gfx950`` (nvcc -arch=sm_90a there, gemm_tuner.py:46) and run as
+  ``./test M 5120 N 5120 K 4096`` with a 30 s limit (gemm_tuner.py:55);
+* the runtime is parsed from ``Average latency (ms) is X`` (gemm_tuner.py:63); compile
+  failure, non-zero exit (the program aborts when its result is wrong), unparsable output
+  and timeout each score ``inf`` and the sweep goes on (gemm_tuner.py:49-72);
+* after every configuration it rewrites ``tuning_results_<timestamp>.json``
+  (``{results:[{params,runtime,success,timestamp}],best_params,best_runtime,timestamp}``)
+  and ``tuning_summary.txt``, and keeps the source of the best configuration so far in
+  ``best_matmul_mi355x.hip`` (gemm_tuner.py:117-164).
+
+Additions: ``prebuild()`` compiles every valid configuration in parallel into
+``<output_dir>/bin`` (hipcc cross-compiles without a GPU, so the slow part can run on a
+build host), ``tune(prebuilt=True)`` then only runs the binaries; ``resume_from`` reloads an
+earlier results JSON and skips what it already holds.
+"""
+from __future__ import annotations
+
+import itertools
+import json
+import os
+import re
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from datetime import datetime
+from pathlib import Path
+from typing import Dict, List, Optional, Tuple
+
+from jinja2 import Template
+
+PKG = Path(__file__).resolve().parent
+if __package__ in (None, ""):
+    sys.path.insert(0, str(PKG.parent))
+    from h100_gemm_amd import kernel_configs as kc      # noqa: E402
+else:
+    from . import kernel_configs as kc
+
+DEFAULT_TEMPLATE = PKG / "template" / "matmul_mi355x.hip.jinja"
+LATENCY_RE = re.compile(r"Average latency \(ms\) is ([\d.]+(?:e[-+]?\d+)?)")
+
+
+def default_compile_command(src: str, exe: str) -> List[str]:
+    return [os.environ.get("HIPCC", "/opt/rocm/bin/hipcc"), "--offload-arch=gfx950", "-O3", "-std=c++17",
+            "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+            "-Wno-unused-command-line-argument", f"-I{PKG / 'csrc'}", f"-I{PKG / 'harness'}",
+            src, "-o", exe, f"-L{PKG / 'lib'}", "-lmi_gemm", f"-Wl,-rpath,{PKG / 'lib'}"]
+
+
+class GemmTuner:
+    def __init__(self, template_file: str = str(DEFAULT_TEMPLATE), output_dir: str = "tuning_results",
+                 work_dir: Optional[str] = None, compile_command=default_compile_command,
+                 bench_args=("M", "5120", "N", "5120", "K", "4096"), timeout: float = 30.0,
+                 resume_from: Optional[str] = None):
+        self.output_dir = Path(output_dir)
+        self.output_dir.mkdir(parents=True, exist_ok=True)
+        self.work_dir = Path(work_dir) if work_dir else self.output_dir
+        self.work_dir.mkdir(parents=True, exist_ok=True)
+        self.compile_command = compile_command
+        self.bench_args = list(bench_args)
+        self.timeout = timeout
+
+        # Define parameter search space
+        self.param_space = {
+            'KIND': ['ring', 'tile'],
+            'BM': [128, 256],
+            'BN': [128, 256],
+            'WM': [2, 4],
+            'WN': [2, 4],
+            'NS': [4],
+            'SWZ': [1],
+            'GROUP': [4, 8, 16],
+            'DTL': [1],
+            'EPI': [1],
+        }
+
+        # Load template
+        with open(template_file, 'r') as f:
+            self.template = Template(f.read())
+
+        self.previous: Dict[str, dict] = {}
+        if resume_from:
+            with open(resume_from, 'r') as f:
+                for r in json.load(f).get('results', []):
+                    self.previous[self.config_key(r['params'])] = r
+
+    @staticmethod
+    def config_key(params: Dict[str, int]) -> str:
+        return json.dumps(params, sort_keys=True)
+
+    @staticmethod
+    def config_name(params: Dict[str, int]) -> str:
+        return kc.config_name(dict(params, OCC=1))
+
+    def generate_code(self, params: Dict[str, int]) -> str:
+        """Generate code with given parameters"""
+        return self.template.render(name=self.config_name(params), **params)
+
+    def _run(self, exe: Path, params) -> Tuple[float, bool]:
+        try:
+            result = subprocess.run([str(Path(exe).resolve())] + self.bench_args, capture_output=True, text=True,
+                                    timeout=self.timeout, cwd=str(self.work_dir))
+            if result.returncode != 0:
+                print(f"Runtime error for parameters: {params}")
+                return float('inf'), False
+            # Extract runtime from output
+            match = LATENCY_RE.search(result.stdout)
+            if match:
+                return float(match.group(1)), True
+            print(f"Could not parse output for parameters: {params}")
+            return float('inf'), False
+        except subprocess.TimeoutExpired:
+            print(f"Timeout for parameters: {params}")
+            return float('inf'), False
+
+    def benchmark_configuration(self, params: Dict[str, int], prebuilt: bool = False) -> Tuple[float, bool]:
+        """Benchmark a single configuration. Returns (runtime, success)"""
+        if prebuilt:
+            exe = self.output_dir / 'bin' / self.config_name(params)
+            if not exe.exists():
+                print(f"Compilation failed for parameters: {params}")
+                return float('inf'), False
+            return self._run(exe, params)
+
+        # Write the generated code to temp.hip
+        src = self.work_dir / 'temp.hip'
+        with open(src, 'w') as f:
+            f.write(self.generate_code(params))
+
+        # If test file exists, remove it
+        test_file = self.work_dir / 'test'
+        if test_file.exists():
+            test_file.unlink()
+
+        # Compile the code
+        compile_result = subprocess.run(self.compile_command(str(src), str(test_file)),
+                                        stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+        if compile_result.returncode != 0 or not test_file.exists():
+            print(f"Compilation failed for parameters: {params}")
+            return float('inf'), False
+
+        # Run the benchmark
+        return self._run(test_file, params)
+
+    def is_valid_configuration(self, params: Dict[str, int]) -> bool:
+        """Check if a parameter configuration is valid"""
+        c = dict(params, OCC=1)
+        if c['KIND'] == 'ring' and (c.get('SWZ', 1) != 1 or c.get('DTL', 1) != 1 or c.get('EPI', 1) != 1):
+            return False            # the ring kernel has one load path and one epilogue
+        if c['KIND'] == 'tile' and c.get('NS', 4) != self.param_space['NS'][0]:
+            return False            # NS is meaningless for the two-stage kernel: keep one copy
+        try:
+            return kc.is_valid_config(c)
+        except KeyError:
+            return False
+
+    def configurations(self) -> List[Dict[str, int]]:
+        combos = [dict(zip(self.param_space.keys(), values))
+                  for values in itertools.product(*self.param_space.values())]
+        return [p for p in combos if self.is_valid_configuration(p)]
+
+    def prebuild(self, jobs: int = 8) -> Dict[str, bool]:
+        """Render and compile every valid configuration into <output_dir>/bin."""
+        bindir = self.output_dir / 'bin'
+        srcdir = self.output_dir / 'src'
+        bindir.mkdir(exist_ok=True)
+        srcdir.mkdir(exist_ok=True)
+
+        def one(params):
+            name = self.config_name(params)
+            src = srcdir / f"{name}.hip"
+            src.write_text(self.generate_code(params))
+            exe = bindir / name
+            r = subprocess.run(self.compile_command(str(src), str(exe)), stdout=subprocess.DEVNULL,
+                               stderr=subprocess.DEVNULL)
+            return name, r.returncode == 0 and exe.exists()
+
+        with ThreadPoolExecutor(max_workers=jobs) as ex:
+            return dict(ex.map(one, self.configurations()))
+
+    def tune(self, prebuilt: bool = False):
+        """Run the tuning process and save results"""
+        results = []
+        best_runtime = float('inf')
+        best_params = None
+
+        # Generate all parameter combinations
+        param_combinations = [dict(zip(self.param_space.keys(), values))
+                              for values in itertools.product(*self.param_space.values())]
+
+        total_configs = len([p for p in param_combinations if self.is_valid_configuration(p)])
+        tested_configs = 0
+
+        for params in param_combinations:
+            if not self.is_valid_configuration(params):
+                continue
+
+            tested_configs += 1
+            print(f"\nTesting configuration {tested_configs}/{total_configs}:")
+            print(params)
+
+            prev = self.previous.get(self.config_key(params))
+            if prev is not None:
+                runtime = prev['runtime'] if prev['success'] else float('inf')
+                success = prev['success']
+                print("(taken from the resumed results)")
+            else:
+                runtime, success = self.benchmark_configuration(params, prebuilt=prebuilt)
+
+            result = {
+                'params': params,
+                'runtime': runtime if success else None,
+                'success': success,
+                'timestamp': datetime.now().isoformat()
+            }
+            results.append(result)
+
+            if success:
+                print(f"Runtime: {runtime:.4f} ms")
+
+            if success and runtime < best_runtime:
+                best_runtime = runtime
+                best_params = params
+                print(f"New best runtime: {best_runtime:.4f} ms")
+
+                # Save the best configuration immediately
+                best_config_file = self.output_dir / 'best_matmul_mi355x.hip'
+                with open(best_config_file, 'w') as f:
+                    f.write(self.generate_code(best_params))
+
+            # Save intermediate results
+            self.save_results(results, best_params, best_runtime)
+
+        return best_params, best_runtime, results
+
+    def save_results(self, results: List[Dict], best_params: Dict[str, int], best_runtime: float):
+        """Save results to disk"""
+        timestamp = datetime.now().strftime('%Y%m%d_%H%M%S')
+
+        # Save detailed results
+        results_file = self.output_dir / f'tuning_results_{timestamp}.json'
+        with open(results_file, 'w') as f:
+            json.dump({
+                'results': results,
+                'best_params': best_params,
+                'best_runtime': best_runtime,
+                'timestamp': timestamp
+            }, f, indent=2)
+
+        # Save summary
+        summary_file = self.output_dir / 'tuning_summary.txt'
+        with open(summary_file, 'w') as f:
+            f.write(f"Tuning completed at: {timestamp}\n")
+            f.write(f"Best runtime: {best_runtime:.4f} ms\n")
+            if best_params:
+                f.write("Best parameters:\n")
+                for key, value in best_params.items():
+                    f.write(f"{key}: {value}\n")
+
+            f.write("\nAll successful configurations:\n")
+            sorted_results = sorted(
+                [r for r in results if r['success']],
+                key=lambda x: x['runtime']
+            )
+            for r in sorted_results:
+                f.write(f"\nRuntime: {r['runtime']:.4f} ms\n")
+                for k, v in r['params'].items():
+                    f.write(f"{k}: {v}\n")
+
+
+def main(argv=None):
+    import argparse
+    ap = argparse.ArgumentParser(description="MI355X GEMM tuner")
+    ap.add_argument("--output-dir", default="tuning_results")
+    ap.add_argument("--prebuild", action="store_true", help="only render + compile every configuration")
+    ap.add_argument("--prebuilt", action="store_true", help="run the binaries a --prebuild left in <output-dir>/bin")
+    ap.add_argument("--resume", default=None, help="results JSON of an earlier run to continue from")
+    ap.add_argument("--shape", nargs=3, type=int, default=[5120, 5120, 4096], metavar=("M", "N", "K"))
+    ap.add_argument("--fill", default=None, choices=["int", "uniform", "normal"])
+    ap.add_argument("-j", "--jobs", type=int, default=8)
+    a = ap.parse_args(argv)
+    bench_args = ["M", str(a.shape[0]), "N", str(a.shape[1]), "K", str(a.shape[2])]
+    if a.fill:
+        bench_args += ["fill", a.fill]
+    tuner = GemmTuner(str(DEFAULT_TEMPLATE), a.output_dir, bench_args=bench_args, resume_from=a.resume)
+    if a.prebuild:
+        built = tuner.prebuild(a.jobs)
+        print(f"compiled {sum(built.values())} of {len(built)} configurations into {tuner.output_dir / 'bin'}")
+        return 0 if all(built.values()) else 1
+    best_params, best_runtime, results = tuner.tune(prebuilt=a.prebuilt)
+
+    if best_params:
+        print("\nTuning completed!")
+        print(f"Best runtime: {best_runtime:.4f} ms")
+        print("Best parameters:")
+        for key, value in best_params.items():
+            print(f"{key}: {value}")
+        print(f"\nResults saved in {a.output_dir} directory")
+    else:
+        print("\nNo valid configuration found!")
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

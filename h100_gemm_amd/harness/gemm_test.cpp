@@ -1,131 +1,18 @@
 // gemm_test.cpp -- the `./test M m N n K k` program of the reference
-// (main() of matmul_h100.cu.jinja:987-1079), on the MI355X library.
-//
-// Same flow: integer random_fill inputs, golden from reference_gpu_gemm, the kernel's
-// output compared with assert_allclose(rtol = 1e-3), then a timed loop, and the same three
-// stdout lines the tuner parses ("Shape ...", "Correct!", "Average latency (ms) is X").
-// Extra key/value pairs, ignored by the reference's parser, select what the six template
-// constants selected there:
-//     cfg <index|name>   kernel configuration (default: the library's choice)
-//     dtype <bf16|fp16>  storage type (default bf16; the reference program is fp16)
-//     iters <n>          timed launches (default 200, as in the reference)
-//     check <0|1>        skip / run the comparison (default 1)
-//     fill <int|uniform|normal>  inputs: the reference's integer random_fill (default),
-//                        seeded U[-1,1), or seeded A ~ N(0,1), B ~ N(0,0.02^2); with the
-//                        last two the comparison uses rtol 2^-6 since sums are inexact
-#include <string>
-
-#include "gemm_host.hpp"
-
-const int testM = 4096;
-const int testN = 4096;
-const int testK = 4096;
-
-template <class T>
-int run(int M, int N, int K, int config, int iters, bool check, const std::string& fill) {
-    using AType = T;
-    using BType = T;
-    using CType = T;
-    using AccumType = float;
-    AccumType alpha = 1.0;
-    AccumType beta = 0.0;
-
-    std::vector<int> AShape = {M, K};
-    std::vector<int> BShape = {N, K};
-    std::vector<int> CShape = {M, N};
-    auto hA = alloc_cpu_tensor<AType>(AShape);
-    auto hB = alloc_cpu_tensor<BType>(BShape);
-    if (fill == "uniform") {
-        uniform_fill(hA, AShape, 69, 1);
-        uniform_fill(hB, BShape, 69, 2);
-    } else if (fill == "normal") {
-        normal_fill(hA, AShape, 69, 1, 1.0f);
-        normal_fill(hB, BShape, 69, 2, 0.02f);
-    } else {
-        random_fill(hA, AShape);
-        random_fill(hB, BShape);
-    }
-    auto hC = alloc_cpu_tensor<CType>(CShape);
-    random_fill(hC, CShape);
-    auto goldenC = alloc_cpu_tensor<CType>(CShape);
-    random_fill(goldenC, CShape);
-    auto dA = alloc_gpu_tensor<AType>(AShape);
-    auto dB = alloc_gpu_tensor<BType>(BShape);
-    auto dgC = alloc_gpu_tensor<CType>(CShape);
-    auto dC = alloc_gpu_tensor<CType>(CShape);
-
-    GPUTimer gpu_timer;
-
-    copy_to_gpu(hA, dA, AShape);
-    copy_to_gpu(hB, dB, BShape);
-    copy_to_gpu(hC, dC, CShape);
-    copy_to_gpu(goldenC, dgC, CShape);
-
-    GemmParams<AType, BType, CType, AccumType> gpu_params(M, N, K, dA, dB, dgC, alpha, beta);
-    GemmParams<AType, BType, CType, AccumType> gpu_kernel_params(M, N, K, dA, dB, dC, alpha, beta);
-
-    if (check) {
-        reference_gpu_gemm(gpu_params);
-        copy_to_cpu(goldenC, dgC, CShape);
-    }
-    gpu_gemm(gpu_kernel_params, config);
-    copy_to_cpu(hC, dC, CShape);
-    if (check) {
-        assert_allclose(hC, goldenC, CShape, /*rtol=*/fill == "int" ? 1e-3f : 0.015625f, /*dump=*/false);
-        std::cout << "Correct!\n";
-    }
-
-    gpu_timer.sync_all();
-    gpu_timer.tick();
-    for (int i = 0; i < iters; ++i) gpu_gemm(gpu_kernel_params, config);
-    gpu_timer.tick();
-    gpu_timer.sync_all();
-    float latency = gpu_timer.report_last_ms() / float(iters);
-    std::cout << "Average latency (ms) is " << latency << "\n";
-    const double tflops = 2.0 * M * N * K / (latency * 1e-3) / 1e12;
-    const int cfg = config == MI_CONFIG_AUTO ? mi_gemm_select_config(mi_dtype_of<T>::value, M, N, K) : config;
-    std::cout << "Config " << mi_gemm_config_name(cfg) << ", " << tflops << " TFLOP/s\n";
-
-    free_cpu_tensor(hA);
-    free_cpu_tensor(hB);
-    free_cpu_tensor(hC);
-    free_cpu_tensor(goldenC);
-    free_gpu_tensor(dA);
-    free_gpu_tensor(dB);
-    free_gpu_tensor(dC);
-    free_gpu_tensor(dgC);
-    return 0;
-}
+// (main() of matmul_h100.cu.jinja:987-1079) over libmi_gemm.so: the kernel is whatever the
+// library's dispatch (or `cfg <index|name>`) selects.  See test_main.hpp for the flow and
+// the extra keys.
+#include "test_main.hpp"
 
 int main(int argc, char** argv) {
-    int M = testM, N = testN, K = testK;
-    int iters = 200, config = MI_CONFIG_AUTO;
-    bool check = true;
-    std::string dtype = "bf16", fill = "int";
-    if (argc > 1) {
-        assert((argc - 1) % 2 == 0);
-        for (int i = 1; i + 1 < argc; i += 2) {
-            std::string keys(argv[i]);
-            char* value = argv[i + 1];
-            if (keys == "M") M = std::atoi(value);
-            else if (keys == "N") N = std::atoi(value);
-            else if (keys == "K") K = std::atoi(value);
-            else if (keys == "iters") iters = std::atoi(value);
-            else if (keys == "check") check = std::atoi(value) != 0;
-            else if (keys == "dtype") dtype = value;
-            else if (keys == "fill") fill = value;
-            else if (keys == "cfg") {
-                char* end = nullptr;
-                long idx = std::strtol(value, &end, 10);
-                config = (end && *end == 0) ? (int)idx : mi_gemm_find_config(value);
-                if (config < 0 || config >= mi_gemm_num_configs()) {
-                    std::cerr << "unknown kernel config " << value << "\n";
-                    return 2;
-                }
-            }
-        }
-    }
-    std::cout << "Shape M=" << M << ", N=" << N << ", K=" << K << "\n";
-    if (dtype == "fp16") return run<half_t>(M, N, K, config, iters, check, fill);
-    return run<bf16>(M, N, K, config, iters, check, fill);
+    TestLaunchFn launch = [](int dtype, int config, int M, int N, int K, const void* A, const void* B,
+                             void* C) { MI_CHECK(mi_gemm_ex(config, dtype, M, N, K, A, B, C, nullptr, nullptr)); };
+    auto label = [](int config) { return std::string(config == MI_CONFIG_AUTO ? "auto" : mi_gemm_config_name(config)); };
+    auto parse = [](const char* value) {
+        char* end = nullptr;
+        long idx = std::strtol(value, &end, 10);
+        int config = (end && *end == 0) ? (int)idx : mi_gemm_find_config(value);
+        return (config < 0 || config >= mi_gemm_num_configs()) ? -1 : config;
+    };
+    return test_main(argc, argv, launch, label, parse);
 }

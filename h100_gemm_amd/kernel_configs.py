@@ -111,6 +111,6 @@ assert len({config_name(c) for c in CONFIGS}) == len(CONFIGS)
 
 # What MI_CONFIG_AUTO resolves to: the big tile when there are enough 256x256 tiles to
 # occupy the chip, the small one otherwise.
-DEFAULT_BIG = CONFIGS[2]
+DEFAULT_BIG = CONFIGS[3]
 DEFAULT_SMALL = CONFIGS[7]
 BIG_MIN_TILES = 64

@@ -66,7 +66,8 @@ int mi_reference_gpu_gemm(int dtype, int M, int N, int K, const void* A, const v
 /* Kernel configuration table (what the tuner sweeps; replaces the six template constants
  * of matmul_h100.cu.jinja:9-14). */
 int mi_gemm_num_configs(void);
-/* Human-readable name, e.g. "t256x256x64_w2x2_rs1_sw1_g8"; NULL if out of range. */
+/* Human-readable name, e.g. "t256x256_w2x2_s1_g4_o1_d1_e1", "r256x256_w2x2_n4_g8" or
+ * "k32x128_n4" (two-stage tile kernel, LDS-ring kernel, decode kernel); NULL if out of range. */
 const char* mi_gemm_config_name(int config);
 /* Index of the config with that name, or -1. */
 int mi_gemm_find_config(const char* name);
@@ -91,6 +92,7 @@ int mi_malloc(void** dptr, size_t bytes);
 int mi_free(void* dptr);
 int mi_memcpy_h2d(void* dst, const void* src, size_t bytes);
 int mi_memcpy_d2h(void* dst, const void* src, size_t bytes);
+int mi_memcpy_d2d(void* dst, const void* src, size_t bytes);
 int mi_memset(void* dst, int value, size_t bytes);
 int mi_device_sync(void);
 int mi_stream_sync(void* stream);
