@@ -49,12 +49,8 @@ def render_sources(configs=None) -> list[Path]:
         p = GEN / f"unit_{c['name']}.hip"
         _write_if_changed(p, unit_t.render(**c))
         units.append(p)
-    names = [c["name"] for c in named]
-    big = names.index(kc.config_name(kc.DEFAULT_BIG)) if hasattr(kc, "DEFAULT_BIG") else 0
-    small = names.index(kc.config_name(kc.DEFAULT_SMALL)) if hasattr(kc, "DEFAULT_SMALL") else len(names) - 1
     _write_if_changed(GEN / "kernel_table.hpp",
-                      table_t.render(configs=named, big_index=big, small_index=small,
-                                     big_min_tiles=getattr(kc, "BIG_MIN_TILES", 64),
+                      table_t.render(configs=named,
                                      skinny_index=sorted((c["BM"], i) for i, c in enumerate(named)
                                                          if c["KIND"] == "skinny")))
     # drop units of configs that no longer exist
@@ -69,7 +65,7 @@ def render_sources(configs=None) -> list[Path]:
 def _stamp(src: Path) -> str:
     h = hashlib.sha1()
     for dep in [src, CSRC / "gemm_kernel.hpp", CSRC / "gemm_launch.hpp", CSRC / "gemm_ring_kernel.hpp",
-                CSRC / "gemm_skinny_kernel.hpp", GEN / "kernel_table.hpp",
+                CSRC / "gemm_skinny_kernel.hpp", CSRC / "gemm_mfma16_kernel.hpp", GEN / "kernel_table.hpp",
                 PKG.parent / "include" / "mi_gemm.h"]:
         h.update(dep.read_bytes())
     h.update(" ".join(HIPFLAGS).encode())

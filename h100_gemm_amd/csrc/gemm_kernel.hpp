@@ -67,9 +67,9 @@ struct GemmArgs {
 //   DTL          1: global -> LDS by direct-to-LDS buffer loads (no staging registers, no
 //                ds_write); 0: global -> registers -> ds_write.  The predicated variant
 //                always stages through registers (it has to mask the K tail there).
-//   EPI          1: the aligned kernel transposes its C tile through LDS and writes whole
-//                256-byte row segments (16 bytes per lane); 0: 8-byte stores straight from
-//                the accumulator layout
+//   EPI          1: the C tile is transposed through LDS and written as whole row segments
+//                (16 bytes per lane); 0: 8-byte stores straight from the accumulator layout
+//                (2-byte stores in the predicated variant when C rows are not 8-byte aligned)
 //   EDGE         predicated variant: any M, N, K and any alignment
 //   DT           storage type (DT_BF16 / DT_FP16)
 template <int BM_, int BN_, int WM_, int WN_, int SWZ_, int GROUP_, int OCC_, int DTL_, int EPI_, bool EDGE_, int DT_>
@@ -78,7 +78,7 @@ struct TileConfig {
     static constexpr int WM = WM_, WN = WN_;
     static constexpr int SWZ = SWZ_, GROUP = GROUP_, OCC = OCC_;
     static constexpr bool DTL = DTL_ != 0 && !EDGE_;
-    static constexpr bool EPI = EPI_ != 0 && !EDGE_;
+    static constexpr bool EPI = EPI_ != 0;
     static constexpr bool EDGE = EDGE_;
     static constexpr int DT = DT_;
     static constexpr int NT = WM * WN * 64;             // threads per workgroup
@@ -232,18 +232,12 @@ gemm_tile_kernel(const GemmArgs p) {
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
     auto gload_a = [&](int kt) __attribute__((always_inline)) {
-#ifdef MI_EXP_NO_GLOAD
-        if (K > 128) return;
-#endif
         const uint32_t kb = (uint32_t)kt * (BK * 2);
 #pragma unroll
         for (int j = 0; j < LA; ++j)
             ga[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrcA, voffA + kb + j * passA, 0, 0);
     };
     auto gload_b = [&](int kt) __attribute__((always_inline)) {
-#ifdef MI_EXP_NO_GLOAD
-        if (K > 128) return;
-#endif
         const uint32_t kb = (uint32_t)kt * (BK * 2);
 #pragma unroll
         for (int j = 0; j < LB; ++j)
@@ -295,18 +289,12 @@ gemm_tile_kernel(const GemmArgs p) {
     auto lds_store_a = [&](int stage) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < LA; ++j) {
-#ifdef MI_EXP_NO_LDS_STORE
-            if (K > 128) { asm volatile("" :: "v"(ga[j])); continue; }
-#endif
             *(u32x4_t*)(lds + stage * A_STAGE + wr_off + j * (RPP * 128)) = ga[j];
         }
     };
     auto lds_store_b = [&](int stage) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < LB; ++j) {
-#ifdef MI_EXP_NO_LDS_STORE
-            if (K > 128) { asm volatile("" :: "v"(gb[j])); continue; }
-#endif
             *(u32x4_t*)(lds + 2 * A_STAGE + stage * B_STAGE + wr_off + j * (RPP * 128)) = gb[j];
         }
     };
@@ -348,9 +336,6 @@ gemm_tile_kernel(const GemmArgs p) {
             (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
         const uint32_t dlds = lds_base + (uint32_t)wave * 1024u;   // + stage + pass * RPP * 128
         auto dma = [&](const __amdgpu_buffer_rsrc_t& rsrc, uint32_t voff, uint32_t dst) __attribute__((always_inline)) {
-#ifdef MI_EXP_NO_DMA
-            if (K > 0) return;
-#endif
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                          :: "s"(dst), "v"(voff), "s"(rsrc) : "memory");
         };
@@ -369,8 +354,6 @@ gemm_tile_kernel(const GemmArgs p) {
         auto vm_barrier = [&]() __attribute__((always_inline)) {
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
         };
-        int kt_dbg = 0;
-        (void)kt_dbg;
         constexpr int NMMA = MI * NI, NFR = MI + NI;
         constexpr int DPM = (LA + LB + NMMA - 1) / NMMA;     // DMA instructions per MFMA slot
         // One MFMA, in the order (i, j) = (idx / NI, idx % NI).
@@ -381,9 +364,6 @@ gemm_tile_kernel(const GemmArgs p) {
         // Fragment r of a k slice, in the order the MFMAs above first need them:
         // A0, B0, B1, .., B(NI-1), A1, .., A(MI-1).
         auto read_one = [&](int stage, int ks, int buf, int r) __attribute__((always_inline)) {
-#ifdef MI_EXP_NO_READS
-            if (kt_dbg > 1) return;
-#endif
             if (r == 0 || r > NI) {
                 const int i = r == 0 ? 0 : r - NI;
                 fa[buf][i] = *(const u32x4_t*)(lds + stage * A_STAGE + a_wave + i * 4096 + rd_off[ks]);
@@ -419,7 +399,6 @@ gemm_tile_kernel(const GemmArgs p) {
             constexpr int nxt = cur ^ 1;
             constexpr bool has1 = decltype(has1_c)::value;
             constexpr bool has2 = decltype(has2_c)::value;
-            kt_dbg = kt;
 #pragma unroll
             for (int ks = 0; ks < 3; ++ks) {
 #pragma unroll
@@ -577,12 +556,20 @@ gemm_tile_kernel(const GemmArgs p) {
     if constexpr (Cfg::EPI) {
         // Through LDS: each wave lays its TM x TN tile out row-major in its own slice of the
         // (now idle) stage buffers, 16-byte chunks XOR-swizzled by the row, then reads rows
-        // back 16 bytes per lane so that one store instruction writes whole TN*2-byte row
-        // segments.  Only the first barrier involves the other waves.
+        // back 16 bytes per lane so that one store instruction writes whole row segments.
+        // Only the first barrier involves the other waves.  The predicated variant masks
+        // rows past M and splits the chunk that straddles N into 2-byte stores; its 16-byte
+        // stores may start at any 2-byte boundary (odd N).
         constexpr int TM = Cfg::TM, TN = Cfg::TN;
         constexpr int CPR = TN / 8;                 // 16-byte chunks per row of the wave tile
-        constexpr int RPI = 64 / CPR;               // rows one read/store instruction covers
+        constexpr bool POW2 = (CPR & (CPR - 1)) == 0;
+        static_assert(CPR % 4 == 0 && (TM * CPR) % 64 == 0, "C staging layout");
         static_assert(TM * TN * 2 * Cfg::WM * Cfg::WN <= Cfg::LDS_BYTES, "staging fits the stage buffers");
+        // bank-conflict-free for 8-byte writes down a column of rows: rows of a power-of-two
+        // width are spread by the row number, 192-byte rows (4 rows = 3 bank rounds) by row / 4
+        auto cswz = [](int row) __attribute__((always_inline)) {
+            return POW2 ? (row & (CPR - 1)) : ((row >> 2) & 3);
+        };
         lds_barrier();                              // every wave is done reading the last stage
         unsigned char* stg = lds + wave * (TM * TN * 2);
 #pragma unroll
@@ -592,7 +579,7 @@ gemm_tile_kernel(const GemmArgs p) {
             for (int j = 0; j < NI; ++j) {
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    const int chunk = (j * 4 + g) ^ (row & (CPR - 1));
+                    const int chunk = (j * 4 + g) ^ cswz(row);
                     u32x2_t w;
                     w[0] = cvt_store2<DT>(acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1]);
                     w[1] = cvt_store2<DT>(acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]);
@@ -601,14 +588,31 @@ gemm_tile_kernel(const GemmArgs p) {
             }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // own writes visible to own reads
-        const int rr = lane / CPR, rc = lane % CPR;
-        const uint32_t cbase =
-            (uint32_t)((wm * TM + rr) * p.ldc + col0 + wn * TN + rc * 8) * 2u;
 #pragma unroll
-        for (int r = 0; r < TM / RPI; ++r) {
-            const int row = r * RPI + rr;
-            const u32x4_t v = *(const u32x4_t*)(stg + row * (TN * 2) + ((rc ^ (row & (CPR - 1))) << 4));
-            __builtin_amdgcn_raw_buffer_store_b128(v, rsrcC, cbase + (uint32_t)(r * RPI * p.ldc) * 2u, 0, 0);
+        for (int r = 0; r < TM * CPR / 64; ++r) {
+            // chunk r*64 + lane of the wave tile, rows first
+            const int idx = r * 64 + lane;
+            const int row = POW2 ? r * (64 / CPR) + lane / CPR : idx / CPR;
+            const int rc = POW2 ? lane % CPR : idx % CPR;
+            const u32x4_t v = *(const u32x4_t*)(stg + row * (TN * 2) + ((rc ^ cswz(row)) << 4));
+            const int m_loc = wm * TM + row;
+            const int n = col0 + wn * TN + rc * 8;
+            const uint32_t off = (uint32_t)(m_loc * p.ldc + n) * 2u;
+            if constexpr (!EDGE) {
+                __builtin_amdgcn_raw_buffer_store_b128(v, rsrcC, off, 0, 0);
+            } else {
+                if (m_loc < rowsA) {
+                    if (n + 7 < N) {
+                        __builtin_amdgcn_raw_buffer_store_b128(v, rsrcC, off, 0, 0);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (n + e < N)
+                                __builtin_amdgcn_raw_buffer_store_b16(
+                                    (uint16_t)(v[e >> 1] >> ((e & 1) * 16)), rsrcC, off + 2 * e, 0, 0);
+                    }
+                }
+            }
         }
     } else {
 #pragma unroll

@@ -1,0 +1,485 @@
+// gemm_mfma16_kernel.hpp -- aligned-shape gfx950 GEMM kernel built on
+// v_mfma_f32_16x16x32_{bf16,f16} with two waves per SIMD (8 waves per workgroup).
+//
+//   C[M,N] = A[M,K] . B[N,K]^T     M % BM == 0, N % BN == 0, K % 128 == 0, 16-byte aligned
+//
+// Why a second MFMA shape: on random bf16 data the chip is power limited, and an MFMA-only
+// loop of 16x16x32 instructions sustains ~2.05 PFLOP/s where 32x32x16 sustains ~1.79 (the
+// 16x16 instruction moves half as many accumulator registers per flop).  The 4-pass
+// instruction needs two waves per SIMD to keep the pipe full, hence 512 threads and a
+// 128 x 64 (or 64 x 128) wave tile with 128 accumulator registers per lane.
+//
+// Everything else follows gemm_kernel.hpp: two LDS stages of one 64-deep K slab each,
+// 128-byte rows with the 16-byte chunks stored at chunk ^ ((row >> 1) & 7), direct-to-LDS
+// buffer loads (inline asm, explicit waits), one barrier per K step, XCD-aware tile order,
+// C tile transposed through LDS and written 16 bytes per lane.  A K step is two 32-deep
+// slices: slice 0 multiplies while the fragments of slice 1 are fetched; after the barrier
+// slice 1 multiplies while slice 0 of the next slab is fetched and the loads of the slab
+// after that are issued.
+//
+// Fragment layout of the 16x16x32 MFMA: lane l holds row (l & 15), k chunk (l >> 4) of the
+// 32-deep slice (8 elements, 16 bytes); result register e of lane l is
+// D[4*(l >> 4) + e][l & 15].  Operands are swapped (B rows as the MFMA "A" matrix) so that a
+// lane holds 4 consecutive n of one m.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <type_traits>
+
+#include "gemm_kernel.hpp"
+
+namespace mi {
+
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+template <int BM_, int BN_, int WM_, int WN_, int GROUP_, int DT_>
+struct Mfma16Config {
+    static constexpr int BM = BM_, BN = BN_, BK = 64;
+    static constexpr int WM = WM_, WN = WN_, GROUP = GROUP_, DT = DT_;
+    static constexpr int NT = WM * WN * 64, NW = WM * WN;
+    static constexpr int TM = BM / WM, TN = BN / WN;
+    static constexpr int MI = TM / 16, NI = TN / 16;
+    static constexpr int RPP = NT / 8;                   // tile rows one pass of all threads loads
+    static constexpr int LA = BM / RPP, LB = BN / RPP;   // load instructions per wave per slab
+    static constexpr int A_STAGE = BM * 128, B_STAGE = BN * 128;
+    static constexpr int LDS_BYTES = 2 * (A_STAGE + B_STAGE);
+    static constexpr int WAVES_PER_EU = NT / 256;
+    static constexpr int NMMA = MI * NI, NFR = MI + NI;
+    static_assert(NT == 512, "two waves per SIMD");
+    static_assert(TM % 16 == 0 && TN % 16 == 0, "wave tile must be a multiple of 16x16");
+    static_assert(BM % RPP == 0 && BN % RPP == 0 && RPP % 16 == 0, "tile rows divide over the threads");
+    static_assert(NFR + 2 * (LA + LB) <= NMMA, "reads and loads each get an MFMA slot");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
+    static_assert(BM * BN * 2 <= LDS_BYTES, "the epilogue stages the C tile in the stage buffers");
+};
+
+template <int DT>
+__device__ __forceinline__ f32x4_t mfma_16x16x32(u32x4_t a, u32x4_t b, f32x4_t c) {
+    if constexpr (DT == DT_BF16) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                      __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+    } else {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a),
+                                                     __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+    }
+}
+
+template <class Cfg, bool TRACE = false>
+__global__ void __launch_bounds__(Cfg::NT)
+__attribute__((amdgpu_waves_per_eu(Cfg::WAVES_PER_EU, Cfg::WAVES_PER_EU)))
+gemm_mfma16_kernel(const GemmArgs p) {
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, WN = Cfg::WN;
+    constexpr int MI = Cfg::MI, NI = Cfg::NI, LA = Cfg::LA, LB = Cfg::LB, RPP = Cfg::RPP;
+    constexpr int A_STAGE = Cfg::A_STAGE, B_STAGE = Cfg::B_STAGE;
+    constexpr int NMMA = Cfg::NMMA, NFR = Cfg::NFR, DT = Cfg::DT;
+    constexpr int TM = Cfg::TM, TN = Cfg::TN;
+
+    // [A stage 0][A stage 1][B stage 0][B stage 1]
+    __shared__ __attribute__((aligned(128))) unsigned char lds[Cfg::LDS_BYTES];
+
+    long long tr_wait = 0, tr_t0 = 0, tr_loop = 0;
+    int tr_cnt = 0;
+    auto tr_now = [&]() __attribute__((always_inline)) { return (long long)__builtin_readcyclecounter(); };
+    if constexpr (TRACE) tr_loop = tr_now();
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+
+    int tm, tn;
+    tile_of_block<Cfg::GROUP>(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, tm, tn);
+    const int row0 = tm * BM, col0 = tn * BN;
+    const int K = p.K;
+    const int KT = K / BK;                               // even (host checks K % 128 == 0)
+
+    const unsigned char* Ab = (const unsigned char*)p.A + (size_t)row0 * p.lda * 2;
+    const unsigned char* Bb = (const unsigned char*)p.B + (size_t)col0 * p.ldb * 2;
+    const uint32_t bytesA = (uint32_t)((BM - 1) * p.lda + K) * 2u;
+    const uint32_t bytesB = (uint32_t)((BN - 1) * p.ldb + K) * 2u;
+    const __amdgpu_buffer_rsrc_t rsrcA = __builtin_amdgcn_make_buffer_rsrc((void*)Ab, 0, (int)bytesA, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrcB = __builtin_amdgcn_make_buffer_rsrc((void*)Bb, 0, (int)bytesB, 0x00020000);
+
+    auto swz = [](int row) __attribute__((always_inline)) { return (row >> 1) & 7; };
+    // direct-to-LDS loads: one instruction fills 8 rows x 128 bytes; lane l lands on chunk
+    // position l & 7 of row l >> 3 and fetches logical chunk (l & 7) ^ swz(row)
+    const int lr = lane >> 3, lc = lane & 7;
+    const int drow = wave * 8 + lr;
+    const int dchunk = lc ^ swz(drow);
+    const uint32_t dvoffA = (uint32_t)(drow * p.lda + dchunk * 8) * 2u;
+    const uint32_t dvoffB = (uint32_t)(drow * p.ldb + dchunk * 8) * 2u;
+    const uint32_t passA = (uint32_t)(RPP * p.lda) * 2u;
+    const uint32_t passB = (uint32_t)(RPP * p.ldb) * 2u;
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
+    const uint32_t dlds = lds_base + (uint32_t)wave * 1024u;
+    auto dma = [&](const __amdgpu_buffer_rsrc_t& rsrc, uint32_t voff, uint32_t dst) __attribute__((always_inline)) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                     :: "s"(dst), "v"(voff), "s"(rsrc) : "memory");
+    };
+    auto dma_one = [&](int kt, int stage, int d) __attribute__((always_inline)) {
+        const uint32_t kb = (uint32_t)kt * (BK * 2);
+        if (d < LA)
+            dma(rsrcA, dvoffA + kb + d * passA, dlds + stage * A_STAGE + d * (RPP * 128));
+        else
+            dma(rsrcB, dvoffB + kb + (d - LA) * passB,
+                dlds + 2 * A_STAGE + stage * B_STAGE + (d - LA) * (RPP * 128));
+    };
+
+    // fragment reads: lane holds row (lane & 15), k chunk 4*ks + (lane >> 4) of the slab
+    const int l16 = lane & 15, q = lane >> 4;
+    int rd_off[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) rd_off[ks] = l16 * 128 + ((((ks << 2) | q) ^ swz(l16)) << 4);
+    const int a_wave = wm * TM * 128;
+    const int b_wave = 2 * A_STAGE + wn * TN * 128;
+
+    u32x4_t fa[2][MI], fb[2][NI];
+    f32x4_t acc[MI][NI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.0f;
+
+    auto mma_one = [&](int buf, int idx) __attribute__((always_inline)) {
+        const int i = idx / NI, j = idx % NI;
+        acc[i][j] = mfma_16x16x32<DT>(fb[buf][j], fa[buf][i], acc[i][j]);
+    };
+    // fragment r of a slice in the order the MFMAs first need them: A0, B0..B(NI-1), A1..
+    auto read_one = [&](int stage, int ks, int buf, int r) __attribute__((always_inline)) {
+        if (r == 0 || r > NI) {
+            const int i = r == 0 ? 0 : r - NI;
+            fa[buf][i] = *(const u32x4_t*)(lds + stage * A_STAGE + a_wave + i * 2048 + rd_off[ks]);
+        } else {
+            const int j = r - 1;
+            fb[buf][j] = *(const u32x4_t*)(lds + stage * B_STAGE + b_wave + j * 2048 + rd_off[ks]);
+        }
+    };
+
+    // ---- prologue: slab 0 -> stage 0, slab 1 -> stage 1 ----
+#pragma unroll
+    for (int d = 0; d < LA + LB; ++d) dma_one(0, 0, d);
+#pragma unroll
+    for (int d = 0; d < LA + LB; ++d) dma_one(1, 1, d);
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"(LA + LB) : "memory");    // slab 0 is in
+#pragma unroll
+    for (int r = 0; r < NFR; ++r) read_one(0, 0, 0, r);
+
+    // load instruction slots of slice 1: every other MFMA after the fragment reads
+    auto kstep = [&](int kt, auto cur_c, auto has1_c, auto has2_c) __attribute__((always_inline)) {
+        constexpr int cur = decltype(cur_c)::value;
+        constexpr int nxt = cur ^ 1;
+        constexpr bool has1 = decltype(has1_c)::value;
+        constexpr bool has2 = decltype(has2_c)::value;
+#pragma unroll
+        for (int idx = 0; idx < NMMA; ++idx) {
+            mma_one(0, idx);
+            if (idx < NFR) read_one(cur, 1, 1, idx);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (has1) {
+            if constexpr (TRACE) tr_t0 = tr_now();
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            if constexpr (TRACE) { tr_wait += tr_now() - tr_t0; ++tr_cnt; }
+        }
+#pragma unroll
+        for (int idx = 0; idx < NMMA; ++idx) {
+            mma_one(1, idx);
+            if constexpr (has1) {
+                if (idx < NFR) read_one(nxt, 0, 0, idx);
+            }
+            if constexpr (has2) {
+                const int d = idx - NFR;
+                if (d >= 0 && (d & 1) == 0 && d / 2 < LA + LB) dma_one(kt + 2, cur, d / 2);
+            }
+
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    using T = std::true_type;
+    using F = std::false_type;
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+    int kt = 0;
+    for (; kt + 2 < KT; kt += 2) {
+        kstep(kt, S0{}, T{}, T{});
+        kstep(kt + 1, S1{}, T{}, T{});
+    }
+    kstep(kt, S0{}, T{}, F{});
+    kstep(kt + 1, S1{}, F{}, F{});
+
+    long long tr_store = 0;
+    if constexpr (TRACE) {
+        tr_store = tr_now();
+        tr_loop = tr_store - tr_loop;
+    }
+    // ---- epilogue: C tile -> storage type -> per-wave LDS staging -> 16-byte row stores ----
+    // acc[i][j][e] of lane l is C[m][n], m = i*16 + (l & 15), n = j*16 + 4*(l >> 4) + e
+    unsigned char* Cb = (unsigned char*)p.C + (size_t)row0 * p.ldc * 2;
+    const uint32_t bytesC = (uint32_t)(BM * p.ldc) * 2u;
+    const __amdgpu_buffer_rsrc_t rsrcC = __builtin_amdgcn_make_buffer_rsrc((void*)Cb, 0, (int)bytesC, 0x00020000);
+    {
+        constexpr int CPR = TN / 8;                 // 16-byte chunks per row of the wave tile
+        constexpr int RPI = 64 / CPR;               // rows per read/store instruction
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");   // all waves done with the last stage
+        unsigned char* stg = lds + wave * (TM * TN * 2);
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+            const int row = i * 16 + l16;
+#pragma unroll
+            for (int j = 0; j < NI; ++j) {
+                const int chunk = (j * 2 + (q >> 1)) ^ (row & (CPR - 1));
+                u32x2_t w;
+                w[0] = cvt_store2<DT>(acc[i][j][0], acc[i][j][1]);
+                w[1] = cvt_store2<DT>(acc[i][j][2], acc[i][j][3]);
+                *(u32x2_t*)(stg + row * (TN * 2) + chunk * 16 + (q & 1) * 8) = w;
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        const int rr = lane / CPR, rc = lane % CPR;
+        const uint32_t cbase = (uint32_t)((wm * TM + rr) * p.ldc + col0 + wn * TN + rc * 8) * 2u;
+#pragma unroll
+        for (int r = 0; r < TM / RPI; ++r) {
+            const int row = r * RPI + rr;
+            const u32x4_t v = *(const u32x4_t*)(stg + row * (TN * 2) + ((rc ^ (row & (CPR - 1))) << 4));
+            __builtin_amdgcn_raw_buffer_store_b128(v, rsrcC, cbase + (uint32_t)(r * RPI * p.ldc) * 2u, 0, 0);
+        }
+    }
+    if constexpr (TRACE) {
+        if (p.DB != nullptr && tid == 0) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            tr_store = tr_now() - tr_store;
+            int* rec = p.DB + 6 * (size_t)blockIdx.x;
+            rec[0] = (int)tr_wait;
+            rec[1] = tr_cnt;
+            rec[2] = (int)tr_loop;
+            rec[3] = KT;
+            rec[4] = (int)tr_store;
+            rec[5] = 1;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Ring variant: K slab = one 32-deep MFMA slice (64-byte LDS rows, chunks stored at
+// chunk ^ ((row >> 2) & 3)), NS stages, loads issued NS slabs ahead and dealt out one per
+// few MFMAs, `vmcnt((NS-2)*L)` waits (never on the youngest loads), one barrier per slab.
+// A slab has NS-1 steps (~3000 cycles at NS = 4) to land instead of ~1.
+template <int BM_, int BN_, int WM_, int WN_, int NS_, int GROUP_, int DT_>
+struct Ring16Config {
+    static constexpr int BM = BM_, BN = BN_, BK = 32;
+    static constexpr int WM = WM_, WN = WN_, NS = NS_, GROUP = GROUP_, DT = DT_;
+    static constexpr int NT = WM * WN * 64, NW = WM * WN;
+    static constexpr int TM = BM / WM, TN = BN / WN;
+    static constexpr int MI = TM / 16, NI = TN / 16;
+    static constexpr int RPP = NW * 16;                  // rows one pass of all waves loads (16 per wave)
+    static constexpr int LA = BM / RPP, LB = BN / RPP;
+    static constexpr int L = LA + LB;
+    static constexpr int A_STAGE = BM * 64, B_STAGE = BN * 64, STAGE = A_STAGE + B_STAGE;
+    static constexpr int LDS_BYTES = NS * STAGE;
+    static constexpr int WAVES_PER_EU = NT / 256;
+    static constexpr int NMMA = MI * NI, NFR = MI + NI;
+    static_assert(NT == 512, "two waves per SIMD");
+    static_assert(TM % 16 == 0 && TN % 16 == 0, "wave tile must be a multiple of 16x16");
+    static_assert(BM % RPP == 0 && BN % RPP == 0, "tile rows divide over the waves");
+    static_assert(NFR + 2 * L <= NMMA, "reads and loads each get an MFMA slot");
+    static_assert(NS >= 3 && NS <= 5 && (NS - 1) * L <= 63, "vmcnt is a 6-bit counter");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
+    static_assert(BM * BN * 2 <= LDS_BYTES, "the epilogue stages the C tile in the ring");
+};
+
+template <class Cfg, bool TRACE = false>
+__global__ void __launch_bounds__(Cfg::NT)
+__attribute__((amdgpu_waves_per_eu(Cfg::WAVES_PER_EU, Cfg::WAVES_PER_EU)))
+gemm_ring16_kernel(const GemmArgs p) {
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::NS, WN = Cfg::WN;
+    constexpr int MI = Cfg::MI, NI = Cfg::NI, LA = Cfg::LA, L = Cfg::L, RPP = Cfg::RPP;
+    constexpr int A_STAGE = Cfg::A_STAGE, STAGE = Cfg::STAGE;
+    constexpr int NMMA = Cfg::NMMA, NFR = Cfg::NFR, DT = Cfg::DT;
+    constexpr int TM = Cfg::TM, TN = Cfg::TN;
+
+    __shared__ __attribute__((aligned(128))) unsigned char lds[Cfg::LDS_BYTES];
+
+    long long tr_wait = 0, tr_t0 = 0, tr_loop = 0;
+    int tr_cnt = 0;
+    auto tr_now = [&]() __attribute__((always_inline)) { return (long long)__builtin_readcyclecounter(); };
+    if constexpr (TRACE) tr_loop = tr_now();
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+
+    int tm, tn;
+    tile_of_block<Cfg::GROUP>(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, tm, tn);
+    const int row0 = tm * BM, col0 = tn * BN;
+    const int K = p.K;
+    const int KT = K / 32;                               // slabs; host checks K % (32*NS) == 0
+
+    const unsigned char* Ab = (const unsigned char*)p.A + (size_t)row0 * p.lda * 2;
+    const unsigned char* Bb = (const unsigned char*)p.B + (size_t)col0 * p.ldb * 2;
+    const uint32_t bytesA = (uint32_t)((BM - 1) * p.lda + K) * 2u;
+    const uint32_t bytesB = (uint32_t)((BN - 1) * p.ldb + K) * 2u;
+    const __amdgpu_buffer_rsrc_t rsrcA = __builtin_amdgcn_make_buffer_rsrc((void*)Ab, 0, (int)bytesA, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrcB = __builtin_amdgcn_make_buffer_rsrc((void*)Bb, 0, (int)bytesB, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrcNone = __builtin_amdgcn_make_buffer_rsrc((void*)Ab, 0, 0, 0x00020000);
+
+    // one load instruction fills 16 rows x 64 bytes: lane l -> row l >> 2, chunk position l & 3
+    const int dr = lane >> 2;
+    const int dchunk = (lane & 3) ^ ((dr >> 2) & 3);
+    const uint32_t dvoffA = (uint32_t)((wave * 16 + dr) * p.lda + dchunk * 8) * 2u;
+    const uint32_t dvoffB = (uint32_t)((wave * 16 + dr) * p.ldb + dchunk * 8) * 2u;
+    const uint32_t passA = (uint32_t)(RPP * p.lda) * 2u;
+    const uint32_t passB = (uint32_t)(RPP * p.ldb) * 2u;
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
+    const uint32_t dlds = lds_base + (uint32_t)wave * 1024u;
+    auto dma = [&](const __amdgpu_buffer_rsrc_t& rsrc, uint32_t voff, uint32_t dst) __attribute__((always_inline)) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                     :: "s"(dst), "v"(voff), "s"(rsrc) : "memory");
+    };
+    auto dma_one = [&](int t, int s, int d) __attribute__((always_inline)) {
+        const uint32_t kb = (uint32_t)t * 64u;
+        const bool live = t < KT;
+        if (d < LA)
+            dma(live ? rsrcA : rsrcNone, dvoffA + kb + d * passA, dlds + s * STAGE + d * (RPP * 64));
+        else
+            dma(live ? rsrcB : rsrcNone, dvoffB + kb + (d - LA) * passB,
+                dlds + s * STAGE + A_STAGE + (d - LA) * (RPP * 64));
+    };
+
+    // fragment reads: lane holds row (lane & 15), chunk (lane >> 4) of the 64-byte row
+    const int l16 = lane & 15, q = lane >> 4;
+    const int rd_off = l16 * 64 + ((q ^ ((l16 >> 2) & 3)) << 4);
+    const int a_wave = wm * TM * 64;
+    const int b_wave = A_STAGE + wn * TN * 64;
+
+    u32x4_t fa[2][MI], fb[2][NI];
+    f32x4_t acc[MI][NI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.0f;
+
+    auto mma_one = [&](int buf, int idx) __attribute__((always_inline)) {
+        const int i = idx / NI, j = idx % NI;
+        acc[i][j] = mfma_16x16x32<DT>(fb[buf][j], fa[buf][i], acc[i][j]);
+    };
+    auto read_one = [&](int s, int buf, int r) __attribute__((always_inline)) {
+        if (r == 0 || r > NI) {
+            const int i = r == 0 ? 0 : r - NI;
+            fa[buf][i] = *(const u32x4_t*)(lds + s * STAGE + a_wave + i * 1024 + rd_off);
+        } else {
+            const int j = r - 1;
+            fb[buf][j] = *(const u32x4_t*)(lds + s * STAGE + b_wave + j * 1024 + rd_off);
+        }
+    };
+
+    // ---- prologue: slabs 0 .. NS-1 ----
+#pragma unroll
+    for (int t = 0; t < NS; ++t)
+#pragma unroll
+        for (int d = 0; d < L; ++d) dma_one(t, t, d);
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"((NS - 1) * L) : "memory");    // slab 0 is in
+#pragma unroll
+    for (int r = 0; r < NFR; ++r) read_one(0, 0, r);
+
+    // One slab.  Fragments of slab t are in register buffer `buf`; stage s held slab t and is
+    // idle (its fragments were fetched during the previous step).
+    //   vmcnt((NS-2)*L) + barrier : slab t+1 has landed for every wave
+    //   32 MFMAs | fetch fragments of slab t+1 | loads of slab t+NS into stage s
+    auto step = [&](int t, auto s_c, auto buf_c) __attribute__((always_inline)) {
+        constexpr int s = decltype(s_c)::value, buf = decltype(buf_c)::value;
+        constexpr int sn = (s + 1) % NS;
+        if constexpr (TRACE) tr_t0 = tr_now();
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" :: "n"((NS - 2) * L) : "memory");
+        if constexpr (TRACE) { tr_wait += tr_now() - tr_t0; ++tr_cnt; }
+#pragma unroll
+        for (int idx = 0; idx < NMMA; ++idx) {
+            mma_one(buf, idx);
+            if (idx < NFR) read_one(sn, buf ^ 1, idx);
+            const int d = idx - NFR;
+            if (d >= 0 && (d & 1) == 0 && d / 2 < L) dma_one(t + NS, s, d / 2);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    using B0 = std::integral_constant<int, 0>;
+    using B1 = std::integral_constant<int, 1>;
+    static_assert(NS == 4, "the step loop below is unrolled for a ring of four");
+    for (int t0 = 0; t0 < KT; t0 += 4) {
+        step(t0, std::integral_constant<int, 0>{}, B0{});
+        step(t0 + 1, std::integral_constant<int, 1>{}, B1{});
+        step(t0 + 2, std::integral_constant<int, 2>{}, B0{});
+        step(t0 + 3, std::integral_constant<int, 3>{}, B1{});
+    }
+    // requests past K are still heading for the ring: drain before reusing it
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+
+    long long tr_store = 0;
+    if constexpr (TRACE) {
+        tr_store = tr_now();
+        tr_loop = tr_store - tr_loop;
+    }
+    unsigned char* Cb = (unsigned char*)p.C + (size_t)row0 * p.ldc * 2;
+    const uint32_t bytesC = (uint32_t)(BM * p.ldc) * 2u;
+    const __amdgpu_buffer_rsrc_t rsrcC = __builtin_amdgcn_make_buffer_rsrc((void*)Cb, 0, (int)bytesC, 0x00020000);
+    {
+        constexpr int CPR = TN / 8;
+        constexpr int RPI = 64 / CPR;
+        unsigned char* stg = lds + wave * (TM * TN * 2);
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+            const int row = i * 16 + l16;
+#pragma unroll
+            for (int j = 0; j < NI; ++j) {
+                const int chunk = (j * 2 + (q >> 1)) ^ (row & (CPR - 1));
+                u32x2_t w;
+                w[0] = cvt_store2<DT>(acc[i][j][0], acc[i][j][1]);
+                w[1] = cvt_store2<DT>(acc[i][j][2], acc[i][j][3]);
+                *(u32x2_t*)(stg + row * (TN * 2) + chunk * 16 + (q & 1) * 8) = w;
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        const int rr = lane / CPR, rc = lane % CPR;
+        const uint32_t cbase = (uint32_t)((wm * TM + rr) * p.ldc + col0 + wn * TN + rc * 8) * 2u;
+#pragma unroll
+        for (int r = 0; r < TM / RPI; ++r) {
+            const int row = r * RPI + rr;
+            const u32x4_t v = *(const u32x4_t*)(stg + row * (TN * 2) + ((rc ^ (row & (CPR - 1))) << 4));
+            __builtin_amdgcn_raw_buffer_store_b128(v, rsrcC, cbase + (uint32_t)(r * RPI * p.ldc) * 2u, 0, 0);
+        }
+    }
+    if constexpr (TRACE) {
+        if (p.DB != nullptr && tid == 0) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            tr_store = tr_now() - tr_store;
+            int* rec = p.DB + 6 * (size_t)blockIdx.x;
+            rec[0] = (int)tr_wait;
+            rec[1] = tr_cnt;
+            rec[2] = (int)tr_loop;
+            rec[3] = KT;
+            rec[4] = (int)tr_store;
+            rec[5] = 1;
+        }
+    }
+}
+
+template <class Cfg, bool TRACE = false>
+hipError_t launch_ring16_kernel(const GemmArgs& args, hipStream_t stream) {
+    const int grid = args.tiles_m * args.tiles_n;
+    hipLaunchKernelGGL((gemm_ring16_kernel<Cfg, TRACE>), dim3(grid), dim3(Cfg::NT), 0, stream, args);
+    return hipGetLastError();
+}
+
+template <class Cfg, bool TRACE = false>
+hipError_t launch_mfma16_kernel(const GemmArgs& args, hipStream_t stream) {
+    const int grid = args.tiles_m * args.tiles_n;
+    hipLaunchKernelGGL((gemm_mfma16_kernel<Cfg, TRACE>), dim3(grid), dim3(Cfg::NT), 0, stream, args);
+    return hipGetLastError();
+}
+
+}  // namespace mi

@@ -177,7 +177,7 @@ int mi_gemm_config_grid(int config, int M, int N, int K) {
 int mi_gemm_select_config(int dtype, int M, int N, int K) {
     (void)dtype;
     // pointer alignment is unknown here: assume the usual 256-byte aligned allocations
-    return mi::select_kernel(M, N, K, M <= 128 && N % 4 == 0 && K % 64 == 0);
+    return mi::select_kernel(M, N, K, M <= 128 && N % 4 == 0 && K % 64 == 0, compute_units());
 }
 
 size_t mi_gemm_trace_words(int M, int N, int K) {
@@ -195,7 +195,7 @@ int mi_gemm_ex(int config, int dtype, int M, int N, int K, const void* A, const 
     int rc = check_args(config, dtype, M, N, K, A, B, C);
     if (rc != MI_OK) return rc;
     const bool streamable = shape_is_streamable(M, N, K, A, B, C);
-    if (config == MI_CONFIG_AUTO) config = mi::select_kernel(M, N, K, streamable);
+    if (config == MI_CONFIG_AUTO) config = mi::select_kernel(M, N, K, streamable, compute_units());
     const mi::KernelEntry& e = mi::kKernels[config];
 
     mi::GemmArgs args;

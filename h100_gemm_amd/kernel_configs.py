@@ -11,9 +11,15 @@ template takes (matmul_h100.cu.jinja:9-14) -- re-cast for CDNA4:
     OCC      workgroups per CU the register budget is sized for
     DTL      1: direct-to-LDS global loads in the aligned kernel, 0: register staged
     KIND     "tile" (two-stage kernel above), "ring" (NS-deep LDS ring, K step 32, aligned
-             shapes; ragged shapes take the predicated tile kernel of the same tile), or
-             "skinny" (split-K streaming kernel for M <= BM, decode shapes)
+             shapes; ragged shapes take the predicated tile kernel of the same tile),
+             "mfma16" / "ring16" (the same two pipelines on the 16x16x32 MFMA with eight
+             waves, csrc/gemm_mfma16_kernel.hpp), or "skinny" (split-K streaming kernel for
+             M <= BM, decode shapes)
     EPI      1: C tile transposed through LDS and written 16 bytes per lane, 0: 8-byte stores
+    EWM, EWN (optional) wave grid of the predicated twin when it differs from WM, WN (the
+             register-staged predicated kernel runs best with eight waves)
+    EFF      (optional) per-CU throughput relative to the 256x256 tile, measured at 8192^3;
+             configs that carry it are the candidates of the automatic shape -> kernel choice
 
 The index of a config in ``CONFIGS`` is its ``config`` number in the C ABI.
 """
@@ -23,10 +29,17 @@ from __future__ import annotations
 def config_name(c: dict) -> str:
     if c["KIND"] == "ring":
         return f"r{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_n{c['NS']}_g{c['GROUP']}"
+    if c["KIND"] == "mfma16":
+        return f"m{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_g{c['GROUP']}"
+    if c["KIND"] == "ring16":
+        return f"q{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_n{c['NS']}_g{c['GROUP']}"
     if c["KIND"] == "skinny":
         return f"k{c['BM']}x{c['BN']}_n{c['NS']}"
-    return (f"t{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_s{c['SWZ']}_g{c['GROUP']}"
+    name = (f"t{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_s{c['SWZ']}_g{c['GROUP']}"
             f"_o{c['OCC']}_d{c['DTL']}_e{c['EPI']}")
+    if (c.get("EWM", c["WM"]), c.get("EWN", c["WN"])) != (c["WM"], c["WN"]):
+        name += f"_x{c['EWM']}x{c['EWN']}"
+    return name
 
 
 def threads(c: dict) -> int:
@@ -34,7 +47,7 @@ def threads(c: dict) -> int:
 
 
 def lds_bytes(c: dict) -> int:
-    if c["KIND"] == "ring":
+    if c["KIND"] in ("ring", "ring16"):
         return c["NS"] * (c["BM"] + c["BN"]) * 64
     if c["KIND"] == "skinny":
         return c["NS"] * (c["BM"] + c["BN"]) * 128
@@ -43,6 +56,12 @@ def lds_bytes(c: dict) -> int:
 
 def is_valid_config(c: dict) -> bool:
     """Static rules of the kernels (mirrored as static_asserts in csrc/)."""
+    if c["KIND"] == "tile" and (c.get("EWM", c["WM"]), c.get("EWN", c["WN"])) != (c["WM"], c["WN"]):
+        twin = dict(c, WM=c["EWM"], WN=c["EWN"], DTL=0)
+        del twin["EWM"], twin["EWN"]
+        main = dict(c)
+        del main["EWM"], main["EWN"]
+        return is_valid_config(twin) and is_valid_config(main)
     if c["KIND"] == "skinny":
         return (c["BM"] % 32 == 0 and c["BN"] % 128 == 0 and c["NS"] >= 2
                 and ((c["BM"] + c["BN"]) // 8) % 4 == 0
@@ -59,6 +78,23 @@ def is_valid_config(c: dict) -> bool:
     if lds_bytes(c) * occ > 160 * 1024:
         return False
     waves_per_simd = max(nt // 256, 1) * occ
+    if c["KIND"] in ("mfma16", "ring16"):
+        # 16x16x32 MFMA kernels: eight waves, 4 accumulator registers per 16x16 tile
+        if nt != 512 or c["BM"] * c["BN"] * 2 > lds_bytes(c):
+            return False
+        mi16, ni16 = 2 * mi, 2 * ni
+        rpp = 64 if c["KIND"] == "mfma16" else 128
+        if c["BM"] % rpp or c["BN"] % rpp:
+            return False
+        l = c["BM"] // rpp + c["BN"] // rpp
+        if c["KIND"] == "ring16" and (c["NS"] != 4 or (c["NS"] - 1) * l > 63):
+            return False
+        tn = c["BN"] // c["WN"]
+        if tn & (tn - 1) or tn < 32:          # the C staging swizzle needs a power-of-two row
+            return False
+        if mi16 + ni16 + 2 * l > mi16 * ni16:
+            return False
+        return mi16 * ni16 * 4 + 2 * (mi16 + ni16) * 4 + 24 <= 256
     if c["KIND"] == "ring":
         rpp = (nt // 64) * 16
         if c["BM"] % rpp or c["BN"] % rpp or c["NS"] != 4:
@@ -78,12 +114,25 @@ def is_valid_config(c: dict) -> bool:
     return regs <= 512 // waves_per_simd
 
 
-def _c(BM, BN, WM, WN, SWZ=1, GROUP=8, OCC=1, DTL=0, EPI=0):
-    return dict(KIND="tile", BM=BM, BN=BN, WM=WM, WN=WN, SWZ=SWZ, GROUP=GROUP, OCC=OCC, DTL=DTL, EPI=EPI)
+def _c(BM, BN, WM, WN, SWZ=1, GROUP=8, OCC=1, DTL=0, EPI=0, EFF=None, EW=None):
+    c = dict(KIND="tile", BM=BM, BN=BN, WM=WM, WN=WN, SWZ=SWZ, GROUP=GROUP, OCC=OCC, DTL=DTL, EPI=EPI)
+    if EW is not None:
+        c["EWM"], c["EWN"] = EW
+    if EFF is not None:
+        c["EFF"] = EFF
+    return c
 
 
 def _r(BM, BN, WM, WN, NS=4, GROUP=8):
     return dict(KIND="ring", BM=BM, BN=BN, WM=WM, WN=WN, NS=NS, GROUP=GROUP)
+
+
+def _m(BM, BN, WM, WN, GROUP=4):
+    return dict(KIND="mfma16", BM=BM, BN=BN, WM=WM, WN=WN, GROUP=GROUP)
+
+
+def _q(BM, BN, WM, WN, NS=4, GROUP=4):
+    return dict(KIND="ring16", BM=BM, BN=BN, WM=WM, WN=WN, NS=NS, GROUP=GROUP)
 
 
 def _k(BM, BN=128, NS=4):
@@ -94,13 +143,20 @@ CONFIGS = [
     _c(256, 256, 2, 2, SWZ=1, GROUP=8),
     _c(256, 256, 2, 2, SWZ=1, GROUP=8, DTL=1),
     _c(256, 256, 2, 2, SWZ=1, GROUP=8, DTL=1, EPI=1),
-    _c(256, 256, 2, 2, SWZ=1, GROUP=4, DTL=1, EPI=1),
+    _c(256, 256, 2, 2, SWZ=1, GROUP=4, DTL=1, EPI=1, EFF=1.0, EW=(2, 4)),
     _c(256, 256, 2, 4, SWZ=1, GROUP=8, DTL=1, EPI=1),
-    _c(256, 128, 2, 2, SWZ=1, GROUP=8, DTL=1, EPI=1),
-    _c(128, 256, 2, 2, SWZ=1, GROUP=8, DTL=1, EPI=1),
-    _c(128, 128, 2, 2, SWZ=1, GROUP=8, OCC=2, DTL=1, EPI=1),
+    _c(256, 192, 2, 2, SWZ=1, GROUP=4, DTL=1, EPI=1),
+    _c(256, 192, 2, 2, SWZ=1, GROUP=4, DTL=1, EPI=1, EFF=0.89, EW=(4, 2)),
+    _c(256, 128, 2, 2, SWZ=1, GROUP=8, DTL=1, EPI=1, EW=(4, 2)),
+    _c(128, 256, 2, 2, SWZ=1, GROUP=8, DTL=1, EPI=1, EW=(2, 4)),
+    _c(256, 128, 2, 2, SWZ=1, GROUP=8, DTL=1, EPI=1, EFF=0.81),
+    _c(128, 256, 2, 2, SWZ=1, GROUP=8, DTL=1, EPI=1, EFF=0.74),
+    _c(128, 128, 2, 2, SWZ=1, GROUP=8, OCC=2, DTL=1, EPI=1, EFF=0.83),
     _r(256, 256, 2, 2),
     _r(256, 256, 2, 4),
+    _m(256, 256, 4, 2),
+    _m(256, 256, 2, 4),
+    _q(256, 256, 4, 2),
     _k(32),
     _k(64),
     _k(128),
@@ -108,9 +164,3 @@ CONFIGS = [
 
 assert all(is_valid_config(c) for c in CONFIGS), [config_name(c) for c in CONFIGS if not is_valid_config(c)]
 assert len({config_name(c) for c in CONFIGS}) == len(CONFIGS)
-
-# What MI_CONFIG_AUTO resolves to: the big tile when there are enough 256x256 tiles to
-# occupy the chip, the small one otherwise.
-DEFAULT_BIG = CONFIGS[3]
-DEFAULT_SMALL = CONFIGS[7]
-BIG_MIN_TILES = 64

@@ -89,7 +89,7 @@ def test_c5_unaligned_full(mi, orc):
 
 # ------------------------------------------------------ every kernel configuration ----
 
-def all_configs(kinds=("tile", "ring")):
+def all_configs(kinds=("tile", "ring", "mfma16", "ring16")):
     from h100_gemm_amd import kernel_configs as kc
     return [i for i, c in enumerate(kc.CONFIGS) if c["KIND"] in kinds]
 
@@ -97,13 +97,13 @@ def all_configs(kinds=("tile", "ring")):
 @pytest.mark.parametrize("config", all_configs())
 def test_every_config_bit_exact_on_integer_fill(mi, orc, config):
     # aligned (512^3: the aligned kernel), and ragged M, N, odd K (the predicated kernel)
-    for M, N, K in [(512, 512, 512), (768, 1280, 1152), (257, 515, 77), (300, 200, 136)]:
+    for M, N, K in [(512, 512, 512), (768, 1536, 1152), (257, 515, 77), (300, 200, 136)]:
         check(mi, orc, M, N, K, "int", config=config, exact=True)
 
 
 @pytest.mark.parametrize("config", all_configs())
 def test_every_config_uniform_within_tolerance(mi, orc, config):
-    for M, N, K in [(1024, 768, 256), (255, 511, 129)]:
+    for M, N, K in [(1024, 768, 256), (255, 511, 129), (513, 391, 320)]:
         check(mi, orc, M, N, K, "uniform", config=config)
 
 

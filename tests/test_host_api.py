@@ -106,6 +106,17 @@ def test_config_table(mi):
     assert kinds == {"skinny"}
     assert kc.CONFIGS[mi.select_config(16, 8192, 8200)]["KIND"] != "skinny"     # K % 64 != 0
     assert kc.CONFIGS[mi.select_config(8192, 8192, 8192)]["KIND"] in ("tile", "ring")
+    # wave quantisation: 256 CUs; 8192^2 fills four rounds of 256x256 tiles, 4095x6143 fills
+    # two rounds of 256x192 tiles exactly (256x256 would leave half of the second round
+    # idle), and 512^2 is a single partial round whatever the tile, so the smallest wins
+    def picked(M, N, K):
+        c = kc.CONFIGS[mi.select_config(M, N, K)]
+        return c["BM"], c["BN"]
+    assert picked(8192, 8192, 8192) == (256, 256)
+    assert picked(8192, 28672, 8192) == (256, 256)
+    assert picked(4095, 6143, 3073) == (256, 192)
+    assert picked(512, 512, 512) == (128, 128)
+    assert all("EFF" in kc.CONFIGS[mi.select_config(M, N, 4096)] for M in (129, 1000, 5000) for N in (100, 3000))
     assert not kc.is_valid_config(dict(KIND="tile", BM=256, BN=256, WM=2, WN=2, SWZ=1, GROUP=8, OCC=2, DTL=0, EPI=0))
     assert not kc.is_valid_config(dict(KIND="tile", BM=96, BN=256, WM=2, WN=2, SWZ=1, GROUP=8, OCC=1, DTL=0, EPI=0))
     assert not kc.is_valid_config(dict(KIND="ring", BM=256, BN=256, WM=2, WN=2, NS=5, GROUP=8))
