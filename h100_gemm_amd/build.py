@@ -37,6 +37,17 @@ def _write_if_changed(path: Path, text: str) -> None:
         path.write_text(text)
 
 
+def _decode_ladder(named) -> list[tuple[int, int]]:
+    """(max M, config index) steps of the automatic choice for decode shapes: per BM the
+    single-pass kernel if there is one, else the split-K kernel."""
+    best = {}
+    for i, c in enumerate(named):
+        if c["KIND"] in ("stream", "skinny"):
+            if c["BM"] not in best or (c["KIND"] == "stream" and named[best[c["BM"]]]["KIND"] != "stream"):
+                best[c["BM"]] = i
+    return sorted(best.items())
+
+
 def render_sources(configs=None) -> list[Path]:
     """Render the per-config units and the kernel table; returns the units' paths."""
     configs = kc.CONFIGS if configs is None else configs
@@ -51,8 +62,7 @@ def render_sources(configs=None) -> list[Path]:
         units.append(p)
     _write_if_changed(GEN / "kernel_table.hpp",
                       table_t.render(configs=named,
-                                     skinny_index=sorted((c["BM"], i) for i, c in enumerate(named)
-                                                         if c["KIND"] == "skinny")))
+                                     skinny_index=_decode_ladder(named)))
     # drop units of configs that no longer exist
     keep = {p.name for p in units}
     for old in GEN.glob("unit_*.hip"):
@@ -65,7 +75,8 @@ def render_sources(configs=None) -> list[Path]:
 def _stamp(src: Path) -> str:
     h = hashlib.sha1()
     for dep in [src, CSRC / "gemm_kernel.hpp", CSRC / "gemm_launch.hpp", CSRC / "gemm_ring_kernel.hpp",
-                CSRC / "gemm_skinny_kernel.hpp", CSRC / "gemm_mfma16_kernel.hpp", GEN / "kernel_table.hpp",
+                CSRC / "gemm_skinny_kernel.hpp", CSRC / "gemm_mfma16_kernel.hpp",
+                CSRC / "gemm_stream_kernel.hpp", GEN / "kernel_table.hpp",
                 PKG.parent / "include" / "mi_gemm.h"]:
         h.update(dep.read_bytes())
     h.update(" ".join(HIPFLAGS).encode())

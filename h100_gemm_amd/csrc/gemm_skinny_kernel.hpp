@@ -4,12 +4,16 @@
 //
 // These shapes are bound by the HBM read of B, not by MFMA, so the kernel is organised
 // around keeping bytes of B in flight on every CU:
-//   * a workgroup owns BN = 128 rows of B and a slice of K (split-K over blockIdx.y), which
-//     gives >= 256 workgroups for N = 8192 while each still amortises its A reads over
-//     128 columns;
+//   * a workgroup owns BN = 128 rows of B and every splits-th 64-deep K slab (split-K over
+//     blockIdx.y, slabs dealt out round-robin), which gives >= 256 workgroups for N = 8192
+//     while each still amortises its A reads over 128 columns;
 //   * B and A slabs (64 k deep, 128-byte rows, XOR-swizzled) go global -> LDS through
 //     direct-to-LDS buffer loads into a ring of NS stages; NS-1 slabs are always in flight;
 //   * one s_barrier per slab; waits are `vmcnt((NS-2)*L)`, never on the youngest loads;
+//   * a workgroup starts its walk over its slabs at one that depends on its position in the
+//     grid and wraps around; together with the round-robin deal this spreads the requests
+//     in flight over every 128-byte position of a row, instead of all workgroups asking for
+//     the same k (the same low address bits, hence the same few HBM channels) at once;
 //   * each of the 4 waves multiplies all BM rows with its own 32 columns
 //     (v_mfma_f32_32x32x16, operands swapped so a lane holds 4 consecutive n);
 //   * with split-K the fp32 partial tiles go to a workspace and splitk_reduce_kernel adds
@@ -34,8 +38,8 @@ struct SkinnyArgs {
     float* ws;        // [splits][M][N] fp32 partials (used when splits > 1)
     int M, N, K;
     int lda, ldb, ldc;
-    int k_per_split;  // multiple of 64
-    int splits;
+    int k_per_split;  // unused by the kernels (kept for the trace / host bookkeeping)
+    int splits;       // <= K / 64
 };
 
 template <int BM_, int BN_, int NS_, int DT_>
@@ -68,17 +72,16 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(const SkinnyArgs p) {
     const int col0 = blockIdx.x * BN;
     const int split = blockIdx.y;
     const int M = p.M, N = p.N, K = p.K;
-    const int k0 = split * p.k_per_split;
-    const int kend = (k0 + p.k_per_split) < K ? (k0 + p.k_per_split) : K;
-    const int KT = (kend - k0) / 64;                         // slabs of this split (>= 1)
+    const int S = p.splits;
+    const int KT = (K / 64 - split + S - 1) / S;             // slabs of this split: split, split+S, .. (>= 1)
 
     const int rowsA = M < BM ? M : BM;
     const int rowsB = (N - col0) < BN ? (N - col0) : BN;
-    const unsigned char* Ab = (const unsigned char*)p.A + (size_t)k0 * 2;
-    const unsigned char* Bb = (const unsigned char*)p.B + ((size_t)col0 * p.ldb + k0) * 2;
-    // descriptors end at the last element this split needs of the last valid row
-    const uint32_t bytesA = (uint32_t)((rowsA - 1) * p.lda + (kend - k0)) * 2u;
-    const uint32_t bytesB = (uint32_t)((rowsB - 1) * p.ldb + (kend - k0)) * 2u;
+    const unsigned char* Ab = (const unsigned char*)p.A;
+    const unsigned char* Bb = (const unsigned char*)p.B + (size_t)col0 * p.ldb * 2;
+    // descriptors end at the last element of the last valid row
+    const uint32_t bytesA = (uint32_t)((rowsA - 1) * p.lda + K) * 2u;
+    const uint32_t bytesB = (uint32_t)((rowsB - 1) * p.ldb + K) * 2u;
     const __amdgpu_buffer_rsrc_t rsrcA = __builtin_amdgcn_make_buffer_rsrc((void*)Ab, 0, (int)bytesA, 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrcB = __builtin_amdgcn_make_buffer_rsrc((void*)Bb, 0, (int)bytesB, 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrcNone = __builtin_amdgcn_make_buffer_rsrc((void*)Ab, 0, 0, 0x00020000);
@@ -95,9 +98,13 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(const SkinnyArgs p) {
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                      :: "s"(dst), "v"(voff), "s"(rsrc) : "memory");
     };
+    // slab t of the loop is this split's slab (t + rot) mod KT, i.e. slab split + S * that of
+    // the matrix; `gs` follows the slab about to be requested
+    int gs = (int)((blockIdx.x * 5u) % (unsigned)KT);
     auto dma_slab = [&](int t, int s) __attribute__((always_inline)) {
         const bool live = t < KT;
-        const uint32_t kb = (uint32_t)t * 128u;
+        const uint32_t kb = (uint32_t)(split + S * gs) * 128u;
+        gs = gs + 1 == KT ? 0 : gs + 1;
 #pragma unroll
         for (int i = 0; i < L; ++i) {
             const int q = wave + i * 4;                      // wave-uniform
@@ -152,7 +159,7 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(const SkinnyArgs p) {
         }
         s = s + 1 == NS ? 0 : s + 1;
     }
-    // loads requested past this split's K range are still heading for the ring
+    // loads requested past this split's last slab are still heading for the ring
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
     // ---- epilogue: lane holds C[m][n..n+3], m = i*32 + (lane & 31), n = 8g + 4*(lane>>5) ----

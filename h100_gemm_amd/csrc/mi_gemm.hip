@@ -159,13 +159,15 @@ int mi_gemm_config_supports(int config, int dtype, int M, int N, int K) {
     if (dtype != MI_DTYPE_BF16 && dtype != MI_DTYPE_FP16) return 0;
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     const mi::KernelEntry& e = mi::kKernels[config];
-    if (e.kind == mi::KIND_SKINNY) return M <= e.BM && N % 4 == 0 && K % 64 == 0;
+    if (e.kind == mi::KIND_SKINNY || e.kind == mi::KIND_STREAM)
+        return M <= e.BM && N % 4 == 0 && K % 64 == 0;
     return e.launch[dtype][1] != nullptr;
 }
 
 int mi_gemm_config_grid(int config, int M, int N, int K) {
     if (config < 0 || config >= mi::kNumKernels || M <= 0 || N <= 0 || K <= 0) return 0;
     const mi::KernelEntry& e = mi::kKernels[config];
+    if (e.kind == mi::KIND_STREAM) return M > e.BM || K % 64 != 0 ? 0 : (N + e.BN - 1) / e.BN;
     if (e.kind == mi::KIND_SKINNY) {
         if (M > e.BM || K % 64 != 0) return 0;
         const int tiles_n = (N + e.BN - 1) / e.BN;
@@ -216,16 +218,24 @@ int mi_gemm_ex(int config, int dtype, int M, int N, int K, const void* A, const 
     args.splits = 1;
     args.k_per_split = K;
 
+    if (e.kind == mi::KIND_STREAM) {
+        if (!streamable || M > e.BM)
+            return fail(MI_ERR_UNSUPPORTED,
+                        "config %s needs M <= %d, N %% 4 == 0, K %% 64 == 0 and 16-byte aligned operands",
+                        e.name, e.BM);
+        hipError_t err = e.launch[dtype][0](args, (hipStream_t)stream);
+        if (err != hipSuccess)
+            return fail(MI_ERR_HIP, "launch of %s failed: %s", e.name, hipGetErrorString(err));
+        return MI_OK;
+    }
     if (e.kind == mi::KIND_SKINNY) {
         if (!streamable || M > e.BM)
             return fail(MI_ERR_UNSUPPORTED,
                         "config %s needs M <= %d, N %% 4 == 0, K %% 64 == 0 and 16-byte aligned operands",
                         e.name, e.BM);
         const int tiles_n = (N + e.BN - 1) / e.BN;
-        args.splits = choose_splits(tiles_n, K, compute_units());
-        const int slabs = K / 64;
-        args.k_per_split = ((slabs + args.splits - 1) / args.splits) * 64;
-        args.splits = (K + args.k_per_split - 1) / args.k_per_split;   // no empty split
+        args.splits = choose_splits(tiles_n, K, compute_units());   // <= K / 64: no empty split
+        args.k_per_split = ((K / 64 + args.splits - 1) / args.splits) * 64;
         if (args.splits > 1) {
             hipError_t we = ensure_workspace((size_t)args.splits * M * N * sizeof(float), &args.ws);
             if (we != hipSuccess)

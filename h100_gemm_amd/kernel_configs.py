@@ -35,6 +35,8 @@ def config_name(c: dict) -> str:
         return f"q{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_n{c['NS']}_g{c['GROUP']}"
     if c["KIND"] == "skinny":
         return f"k{c['BM']}x{c['BN']}_n{c['NS']}"
+    if c["KIND"] == "stream":
+        return f"s{c['BM']}x{c['BN']}_n{c['NS']}"
     name = (f"t{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_s{c['SWZ']}_g{c['GROUP']}"
             f"_o{c['OCC']}_d{c['DTL']}_e{c['EPI']}")
     if (c.get("EWM", c["WM"]), c.get("EWN", c["WN"])) != (c["WM"], c["WN"]):
@@ -43,7 +45,7 @@ def config_name(c: dict) -> str:
 
 
 def threads(c: dict) -> int:
-    return 256 if c["KIND"] == "skinny" else c["WM"] * c["WN"] * 64
+    return 256 if c["KIND"] in ("skinny", "stream") else c["WM"] * c["WN"] * 64
 
 
 def lds_bytes(c: dict) -> int:
@@ -51,6 +53,8 @@ def lds_bytes(c: dict) -> int:
         return c["NS"] * (c["BM"] + c["BN"]) * 64
     if c["KIND"] == "skinny":
         return c["NS"] * (c["BM"] + c["BN"]) * 128
+    if c["KIND"] == "stream":
+        return 4 * c["NS"] * (c["BM"] + c["BN"]) * 128
     return 2 * (c["BM"] + c["BN"]) * 128
 
 
@@ -62,6 +66,11 @@ def is_valid_config(c: dict) -> bool:
         main = dict(c)
         del main["EWM"], main["EWN"]
         return is_valid_config(twin) and is_valid_config(main)
+    if c["KIND"] == "stream":
+        return (c["BM"] in (16, 32, 64) and c["BN"] == 32 and c["NS"] >= 2
+                and (c["NS"] - 1) * ((c["BM"] + c["BN"]) // 8) <= 63
+                and c["NS"] * (c["BM"] + c["BN"]) * 128 >= max(c["BM"], 32) * 128
+                and lds_bytes(c) <= 160 * 1024)
     if c["KIND"] == "skinny":
         return (c["BM"] % 32 == 0 and c["BN"] % 128 == 0 and c["NS"] >= 2
                 and ((c["BM"] + c["BN"]) // 8) % 4 == 0
@@ -135,6 +144,10 @@ def _q(BM, BN, WM, WN, NS=4, GROUP=4):
     return dict(KIND="ring16", BM=BM, BN=BN, WM=WM, WN=WN, NS=NS, GROUP=GROUP)
 
 
+def _s(BM, NS):
+    return dict(KIND="stream", BM=BM, BN=32, NS=NS)
+
+
 def _k(BM, BN=128, NS=4):
     return dict(KIND="skinny", BM=BM, BN=BN, NS=NS)
 
@@ -157,6 +170,9 @@ CONFIGS = [
     _m(256, 256, 4, 2),
     _m(256, 256, 2, 4),
     _q(256, 256, 4, 2),
+    _s(16, 5),
+    _s(32, 4),
+    _s(64, 3),
     _k(32),
     _k(64),
     _k(128),

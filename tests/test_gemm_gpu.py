@@ -109,7 +109,7 @@ def test_every_config_uniform_within_tolerance(mi, orc, config):
 
 # ------------------------------------------------ decode (split-K streaming) kernels ----
 
-@pytest.mark.parametrize("config", all_configs(("skinny",)))
+@pytest.mark.parametrize("config", all_configs(("skinny", "stream")))
 def test_decode_kernels(mi, orc, config):
     from h100_gemm_amd import kernel_configs as kc
     bm = kc.CONFIGS[config]["BM"]
@@ -134,11 +134,12 @@ def test_decode_dispatch_and_determinism(mi, orc):
     # otherwise -- same answers either way
     for M, N, K in [(16, 8192, 8192), (100, 4100, 2112), (128, 8190, 1024), (5, 256, 8200), (128, 8192, 8192)]:
         check(mi, orc, M, N, K, "int", exact=True)
-    A, B = make_inputs(orc, 64, 8192, 8192, "normal")
-    d = Dev(mi, A, B, 64, 8192)
-    C0 = d.run(8192)
-    for _ in range(3):
-        assert (d.run(8192) == C0).all()          # fixed split order: bit-reproducible
+    for M in (16, 64):                            # single-pass kernel, split-K kernel
+        A, B = make_inputs(orc, M, 8192, 8192, "normal")
+        d = Dev(mi, A, B, M, 8192)
+        C0 = d.run(8192)
+        for _ in range(3):
+            assert (d.run(8192) == C0).all()      # fixed summation order: bit-reproducible
 
 
 # --------------------------------------------------------------------- edge cases ----

@@ -84,7 +84,7 @@ def test_config_table(mi):
     for i, c in enumerate(kc.CONFIGS):
         assert L.mi_gemm_config_lds_bytes(i) == kc.lds_bytes(c) <= 160 * 1024
         assert kc.is_valid_config(c)
-        if c["KIND"] == "skinny":
+        if c["KIND"] in ("skinny", "stream"):
             # decode kernels: M <= BM, whole 64-deep K slabs, N a multiple of 4; no ragged twin
             assert L.mi_gemm_config_supports(i, 0, c["BM"], 8192, 8192) == 1
             assert L.mi_gemm_config_supports(i, 0, c["BM"] + 1, 8192, 8192) == 0
@@ -103,7 +103,7 @@ def test_config_table(mi):
         assert 0 <= mi.select_config(M, N, K) < n
         assert L.mi_gemm_trace_words(M, N, K) >= 7
     kinds = {kc.CONFIGS[mi.select_config(M, 8192, 8192)]["KIND"] for M in (16, 64, 128)}
-    assert kinds == {"skinny"}
+    assert kinds <= {"skinny", "stream"}
     assert kc.CONFIGS[mi.select_config(16, 8192, 8200)]["KIND"] != "skinny"     # K % 64 != 0
     assert kc.CONFIGS[mi.select_config(8192, 8192, 8192)]["KIND"] in ("tile", "ring")
     # wave quantisation: 256 CUs; 8192^2 fills four rounds of 256x256 tiles, 4095x6143 fills
