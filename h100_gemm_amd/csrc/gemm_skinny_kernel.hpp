@@ -1,4 +1,4 @@
-// gemm_skinny_kernel.hpp -- gfx950 GEMM kernel for decode-shaped problems (M <= 128):
+// gemm_skinny_kernel.hpp -- gfx950 split-K GEMM kernel for decode-shaped problems (M <= 128):
 //
 //   C[M,N] = A[M,K] . B[N,K]^T     M small, B (the weights) streamed once from HBM
 //
@@ -7,18 +7,23 @@
 //   * a workgroup owns BN = 128 rows of B and every splits-th 64-deep K slab (split-K over
 //     blockIdx.y, slabs dealt out round-robin), which gives >= 256 workgroups for N = 8192
 //     while each still amortises its A reads over 128 columns;
-//   * B and A slabs (64 k deep, 128-byte rows, XOR-swizzled) go global -> LDS through
-//     direct-to-LDS buffer loads into a ring of NS stages; NS-1 slabs are always in flight;
-//   * one s_barrier per slab; waits are `vmcnt((NS-2)*L)`, never on the youngest loads;
+//   * B and A slabs (128-byte rows, XOR-swizzled) go global -> LDS through direct-to-LDS
+//     buffer loads into a ring of NS stages; at the top of a slab the next one has already
+//     landed and NS-3 more are in flight, a further one is requested during the slab;
 //   * a workgroup starts its walk over its slabs at one that depends on its position in the
 //     grid and wraps around; together with the round-robin deal this spreads the requests
 //     in flight over every 128-byte position of a row, instead of all workgroups asking for
 //     the same k (the same low address bits, hence the same few HBM channels) at once;
-//   * each of the 4 waves multiplies all BM rows with its own 32 columns
-//     (v_mfma_f32_32x32x16, operands swapped so a lane holds 4 consecutive n);
+//   * one s_barrier per slab; waits are `vmcnt((NS-3)*L)`, never on the youngest loads;
+//   * 4 waves in a WM x WN grid, v_mfma_f32_32x32x16 with the operands swapped so that a
+//     lane holds 4 consecutive n; the fragments of k slice ks+1 (or of slice 0 of the next
+//     slab) are fetched while slice ks multiplies, dealt out over the MFMA slots;
 //   * with split-K the fp32 partial tiles go to a workspace and splitk_reduce_kernel adds
-//     them in a fixed order (so results are reproducible) and rounds once to the storage
-//     type; without split-K the tile is rounded and stored directly.
+//     them in split order -- a fixed order, so results are reproducible -- and rounds once
+//     to the storage type; without split-K the tile is rounded and stored directly.  (Adding
+//     the partials in the last workgroup to arrive instead was measured 3x slower: the
+//     device-scope fences it needs write back and invalidate the whole L2 of the XCD once
+//     per workgroup.)
 // The reference has no counterpart: its kernels assert M % 128 == 0 (matmul_utils.cuh:362,
 // 386-387).  Rows of A past M are never fetched (the buffer descriptor ends at row M-1 and
 // out-of-range loads return zero).
@@ -34,41 +39,44 @@ namespace mi {
 struct SkinnyArgs {
     const void* A;
     const void* B;
-    void* C;          // storage-type output (used when splits == 1)
-    float* ws;        // [splits][M][N] fp32 partials (used when splits > 1)
+    void* C;              // storage-type output
+    float* ws;            // [splits][M][N] fp32 partials (used when splits > 1)
     int M, N, K;
     int lda, ldb, ldc;
-    int k_per_split;  // unused by the kernels (kept for the trace / host bookkeeping)
-    int splits;       // <= K / 64
+    int k_per_split;      // unused by the kernels (host bookkeeping)
+    int splits;           // <= K / 64
 };
 
 template <int BM_, int BN_, int NS_, int DT_>
 struct SkinnyConfig {
     static constexpr int BM = BM_, BN = BN_, NS = NS_, DT = DT_;
     static constexpr int NT = 256, NW = 4;
-    static constexpr int MI = BM / 32;                       // 32-row MFMA blocks
-    static constexpr int TN = BN / NW;                       // columns per wave
-    static constexpr int NI = TN / 32;
+    static constexpr int WM = BM >= 64 ? 2 : 1, WN = NW / WM;   // wave grid
+    static constexpr int TM = BM / WM, TN = BN / WN;         // wave tile
+    static constexpr int MI = TM / 32, NI = TN / 32;
+    static constexpr int NMMA = MI * NI, NFR = MI + NI;
     static constexpr int ROWS = BM + BN;                     // rows of one stage: A then B
     static constexpr int STAGE = ROWS * 128;
     static constexpr int L = ROWS / 8 / NW;                  // load instructions per wave per slab
     static constexpr int LDS_BYTES = NS * STAGE;
-    static_assert(BM % 32 == 0 && TN % 32 == 0, "MFMA blocks are 32x32");
+    static_assert(TM % 32 == 0 && TN % 32 == 0, "MFMA blocks are 32x32");
     static_assert((ROWS / 8) % NW == 0, "load instructions divide over the waves");
-    static_assert(NS >= 2 && (NS - 1) * L <= 63, "vmcnt is a 6-bit counter");
+    static_assert(NS >= 3 && (NS - 1) * L <= 63, "vmcnt is a 6-bit counter");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
 };
 
 template <class Cfg>
 __global__ void __launch_bounds__(256) gemm_skinny_kernel(const SkinnyArgs p) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::NS, DT = Cfg::DT;
-    constexpr int MI = Cfg::MI, NI = Cfg::NI, TN = Cfg::TN, L = Cfg::L, STAGE = Cfg::STAGE;
+    constexpr int MI = Cfg::MI, NI = Cfg::NI, TM = Cfg::TM, TN = Cfg::TN, L = Cfg::L, STAGE = Cfg::STAGE;
+    constexpr int NMMA = Cfg::NMMA, NFR = Cfg::NFR;
 
     __shared__ __attribute__((aligned(128))) unsigned char lds[Cfg::LDS_BYTES];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
     const int col0 = blockIdx.x * BN;
     const int split = blockIdx.y;
     const int M = p.M, N = p.N, K = p.K;
@@ -94,28 +102,38 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(const SkinnyArgs p) {
     const int lr = lane >> 3, lc = lane & 7;
     auto swz = [](int row) __attribute__((always_inline)) { return (row >> 1) & 7; };
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
-    auto dma = [&](const __amdgpu_buffer_rsrc_t& rsrc, uint32_t voff, uint32_t dst) __attribute__((always_inline)) {
+    auto dma = [](__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t dst) __attribute__((always_inline)) {
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                      :: "s"(dst), "v"(voff), "s"(rsrc) : "memory");
     };
-    // slab t of the loop is this split's slab (t + rot) mod KT, i.e. slab split + S * that of
-    // the matrix; `gs` follows the slab about to be requested
-    int gs = (int)((blockIdx.x * 5u) % (unsigned)KT);
-    auto dma_slab = [&](int t, int s) __attribute__((always_inline)) {
-        const bool live = t < KT;
-        const uint32_t kb = (uint32_t)(split + S * gs) * 128u;
-        gs = gs + 1 == KT ? 0 : gs + 1;
+    uint32_t voff[L];
 #pragma unroll
-        for (int i = 0; i < L; ++i) {
-            const int q = wave + i * 4;                      // wave-uniform
-            const int row = q * 8 + lr;                      // stage row of this lane
-            const int chunk = lc ^ swz(row);
-            const uint32_t dst = lds_base + (uint32_t)(s * STAGE + q * 1024);
-            if (q * 8 < BM) {
-                dma(live ? rsrcA : rsrcNone, (uint32_t)(row * p.lda + chunk * 8) * 2u + kb, dst);
-            } else {
-                dma(live ? rsrcB : rsrcNone, (uint32_t)((row - BM) * p.ldb + chunk * 8) * 2u + kb, dst);
-            }
+    for (int i = 0; i < L; ++i) {
+        const int q = wave + i * 4;                          // wave-uniform
+        const int row = q * 8 + lr;                          // stage row of this lane
+        const int chunk = lc ^ swz(row);
+        voff[i] = q * 8 < BM ? (uint32_t)(row * p.lda + chunk * 8) * 2u
+                             : (uint32_t)((row - BM) * p.ldb + chunk * 8) * 2u;
+    }
+    // Slab t of the loop is this split's slab (t + rot) mod KT, i.e. slab split + S * that of
+    // the matrix.  `gs` follows the slab being requested, `issued` counts requested slabs.
+    int gs = (int)((blockIdx.x * 5u) % (unsigned)KT);
+    int issued = 0;
+    uint32_t kb_cur = 0;
+    bool live_cur = false;
+    auto begin_slab = [&]() __attribute__((always_inline)) {
+        live_cur = issued < KT;
+        kb_cur = (uint32_t)(split + S * gs) * 128u;
+        gs = gs + 1 == KT ? 0 : gs + 1;
+        ++issued;
+    };
+    auto dma_one = [&](int s, int i) __attribute__((always_inline)) {
+        const int q = wave + i * 4;
+        const uint32_t dst = lds_base + (uint32_t)(s * STAGE + q * 1024);
+        if (q * 8 < BM) {
+            dma(live_cur ? rsrcA : rsrcNone, voff[i] + kb_cur, dst);
+        } else {
+            dma(live_cur ? rsrcB : rsrcNone, voff[i] + kb_cur, dst);
         }
     };
 
@@ -124,8 +142,10 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(const SkinnyArgs p) {
     int rd_off[4];
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) rd_off[ks] = l32 * 128 + ((((ks << 1) | hi) ^ swz(l32)) << 4);
-    const int b_wave = (BM + wave * TN) * 128;
+    const int a_wave = wm * TM * 128;
+    const int b_wave = (BM + wn * TN) * 128;
 
+    u32x4_t fa[2][MI], fb[2][NI];
     f32x16_t acc[MI][NI];
 #pragma unroll
     for (int i = 0; i < MI; ++i)
@@ -134,47 +154,77 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(const SkinnyArgs p) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-    // ---- prologue: slabs 0 .. NS-2 in flight ----
+    auto mma_one = [&](int buf, int idx) __attribute__((always_inline)) {
+        const int i = idx / NI, j = idx % NI;
+        acc[i][j] = mfma_32x32x16<DT>(fb[buf][j], fa[buf][i], acc[i][j]);
+    };
+    // fragment r of a k slice in the order the MFMAs first need them: A0, B0..B(NI-1), A1..
+    auto read_one = [&](const unsigned char* st, int ks, int buf, int r) __attribute__((always_inline)) {
+        if (r == 0 || r > NI) {
+            const int i = r == 0 ? 0 : r - NI;
+            fa[buf][i] = *(const u32x4_t*)(st + a_wave + i * 4096 + rd_off[ks]);
+        } else {
+            const int j = r - 1;
+            fb[buf][j] = *(const u32x4_t*)(st + b_wave + j * 4096 + rd_off[ks]);
+        }
+    };
+    constexpr int RPS = (NFR + NMMA - 1) / NMMA;             // LDS reads per MFMA slot
+    constexpr int DPS = (L + 4 * NMMA - 1) / (4 * NMMA);     // load instructions per MFMA slot
+
+    // ---- prologue: slabs 0 .. NS-2 requested, slab 0 landed, its first fragments fetched ----
 #pragma unroll
-    for (int t = 0; t < NS - 1; ++t) dma_slab(t, t);
+    for (int t = 0; t < NS - 1; ++t) {
+        begin_slab();
+#pragma unroll
+        for (int i = 0; i < L; ++i) dma_one(t, i);
+    }
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"((NS - 2) * L) : "memory");
+#pragma unroll
+    for (int r = 0; r < NFR; ++r) read_one(lds, 0, 0, r);
 
     int s = 0;
     for (int t = 0; t < KT; ++t) {
-        // slab t has landed for every wave, and every wave is done with slab t-1
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" :: "n"((NS - 2) * L) : "memory");
-        // refill the stage that slab t-1 occupied
-        dma_slab(t + NS - 1, s == 0 ? NS - 1 : s - 1);
+        const int sn = s + 1 == NS ? 0 : s + 1;              // stage of slab t+1
+        const int sf = s == 0 ? NS - 1 : s - 1;              // stage of slab t-1: refilled now
+        // slab t+1 has landed for every wave, every wave is done with slab t-1
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" :: "n"((NS - 3) * L) : "memory");
+        begin_slab();
         const unsigned char* st = lds + s * STAGE;
+        const unsigned char* stn = lds + sn * STAGE;
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
-            u32x4_t fa[MI], fb[NI];
 #pragma unroll
-            for (int i = 0; i < MI; ++i) fa[i] = *(const u32x4_t*)(st + i * 4096 + rd_off[ks]);
+            for (int idx = 0; idx < NMMA; ++idx) {
+                mma_one(ks & 1, idx);
 #pragma unroll
-            for (int j = 0; j < NI; ++j) fb[j] = *(const u32x4_t*)(st + b_wave + j * 4096 + rd_off[ks]);
+                for (int r = idx * RPS; r < (idx + 1) * RPS && r < NFR; ++r) {
+                    if (ks < 3) read_one(st, ks + 1, (ks + 1) & 1, r);
+                    else read_one(stn, 0, 0, r);             // after the last slab: stale bytes, never used
+                }
 #pragma unroll
-            for (int i = 0; i < MI; ++i)
-#pragma unroll
-                for (int j = 0; j < NI; ++j) acc[i][j] = mfma_32x32x16<DT>(fb[j], fa[i], acc[i][j]);
+                for (int d = (ks * NMMA + idx) * DPS; d < (ks * NMMA + idx + 1) * DPS && d < L; ++d)
+                    dma_one(sf, d);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
-        s = s + 1 == NS ? 0 : s + 1;
+        s = sn;
     }
     // loads requested past this split's last slab are still heading for the ring
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
 
     // ---- epilogue: lane holds C[m][n..n+3], m = i*32 + (lane & 31), n = 8g + 4*(lane>>5) ----
-    if (p.splits == 1) {
+    if (S == 1) {
         unsigned char* Cb = (unsigned char*)p.C;
         const __amdgpu_buffer_rsrc_t rsrcC =
             __builtin_amdgcn_make_buffer_rsrc((void*)Cb, 0, (int)((uint32_t)(M * p.ldc) * 2u), 0x00020000);
 #pragma unroll
         for (int i = 0; i < MI; ++i) {
-            const int m = i * 32 + l32;
+            const int m = wm * TM + i * 32 + l32;
 #pragma unroll
             for (int j = 0; j < NI; ++j)
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    const int n = col0 + wave * TN + j * 32 + g * 8 + hi * 4;
+                    const int n = col0 + wn * TN + j * 32 + g * 8 + hi * 4;
                     if (m < M && n < N) {           // N % 4 == 0 is a launch precondition
                         u32x2_t w;
                         w[0] = cvt_store2<DT>(acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1]);
@@ -183,23 +233,23 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(const SkinnyArgs p) {
                     }
                 }
         }
-    } else {
-        float* P = p.ws + (size_t)split * M * N;
+        return;
+    }
+    float* P = p.ws + (size_t)split * M * N;
 #pragma unroll
-        for (int i = 0; i < MI; ++i) {
-            const int m = i * 32 + l32;
+    for (int i = 0; i < MI; ++i) {
+        const int m = wm * TM + i * 32 + l32;
 #pragma unroll
-            for (int j = 0; j < NI; ++j)
+        for (int j = 0; j < NI; ++j)
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int n = col0 + wave * TN + j * 32 + g * 8 + hi * 4;
-                    if (m < M && n < N) {
-                        float4 v = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2],
-                                    acc[i][j][g * 4 + 3]};
-                        *(float4*)(P + (size_t)m * N + n) = v;
-                    }
+            for (int g = 0; g < 4; ++g) {
+                const int n = col0 + wn * TN + j * 32 + g * 8 + hi * 4;
+                if (m < M && n < N) {
+                    float4 v = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2],
+                                acc[i][j][g * 4 + 3]};
+                    *(float4*)(P + (size_t)m * N + n) = v;
                 }
-        }
+            }
     }
 }
 

@@ -72,7 +72,7 @@ def is_valid_config(c: dict) -> bool:
                 and c["NS"] * (c["BM"] + c["BN"]) * 128 >= max(c["BM"], 32) * 128
                 and lds_bytes(c) <= 160 * 1024)
     if c["KIND"] == "skinny":
-        return (c["BM"] % 32 == 0 and c["BN"] % 128 == 0 and c["NS"] >= 2
+        return (c["BM"] % 32 == 0 and c["BN"] % 128 == 0 and c["NS"] >= 3
                 and ((c["BM"] + c["BN"]) // 8) % 4 == 0
                 and (c["NS"] - 1) * ((c["BM"] + c["BN"]) // 32) <= 63
                 and lds_bytes(c) <= 160 * 1024)
@@ -173,9 +173,9 @@ CONFIGS = [
     _s(16, 5),
     _s(32, 4),
     _s(64, 3),
-    _k(32),
-    _k(64),
-    _k(128),
+    _k(32, NS=4),
+    _k(64, NS=6),
+    _k(128, NS=5),
 ]
 
 assert all(is_valid_config(c) for c in CONFIGS), [config_name(c) for c in CONFIGS if not is_valid_config(c)]
