@@ -62,6 +62,9 @@ def render_sources(configs=None) -> list[Path]:
         units.append(p)
     _write_if_changed(GEN / "kernel_table.hpp",
                       table_t.render(configs=named,
+                                     tuned=[(m, n, k, [c["name"] for c in named].index(nm))
+                                            for (m, n, k), nm in sorted(getattr(kc, "TUNED_SHAPES", {}).items())
+                                            if nm in [c["name"] for c in named]],
                                      skinny_index=_decode_ladder(named)))
     # drop units of configs that no longer exist
     keep = {p.name for p in units}
