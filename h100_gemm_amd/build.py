@@ -38,14 +38,10 @@ def _write_if_changed(path: Path, text: str) -> None:
 
 
 def _decode_ladder(named) -> list[tuple[int, int]]:
-    """(max M, config index) steps of the automatic choice for decode shapes: per BM the
-    single-pass kernel if there is one, else the split-K kernel."""
-    best = {}
-    for i, c in enumerate(named):
-        if c["KIND"] in ("stream", "skinny"):
-            if c["BM"] not in best or (c["KIND"] == "stream" and named[best[c["BM"]]]["KIND"] != "stream"):
-                best[c["BM"]] = i
-    return sorted(best.items())
+    """(max M, config index) steps of the automatic choice for decode shapes."""
+    names = [c["name"] for c in named]
+    ladder = getattr(kc, "DECODE_LADDER", [])
+    return [(m, names.index(n)) for m, n in ladder if n in names]
 
 
 def render_sources(configs=None) -> list[Path]:

@@ -53,12 +53,15 @@ bool shape_is_streamable(int M, int N, int K, const void* A, const void* B, cons
            (((uintptr_t)C & 7u) == 0);
 }
 
-// Split-K geometry for a decode launch: aim at two workgroups per CU, keep at least four
-// K slabs per split.  MI_GEMM_SPLITK=<n> overrides (tuning aid).
-int choose_splits(int tiles_n, int K, int cus) {
+// Split-K geometry for a decode launch.  These kernels are bound by memory latency, not by
+// CU count: about three quarters of the workgroups the chip can hold at once measured best
+// (8192 x 8192 weights, M = 64 and 128: 3 splits 30 / 38 us, 4 splits 35 / 41 us, 8 splits
+// 39 / 46 us).  At least four K slabs per split.  MI_GEMM_SPLITK=<n> overrides (tuning aid).
+int choose_splits(int tiles_n, int K, int cus, int lds_bytes) {
     static const int env = [] { const char* s = getenv("MI_GEMM_SPLITK"); return s ? atoi(s) : 0; }();
     const int slabs = K / 64;
-    int splits = env > 0 ? env : (2 * cus + tiles_n - 1) / tiles_n;
+    const int resident = cus * (lds_bytes > 0 && 160 * 1024 / lds_bytes > 1 ? 160 * 1024 / lds_bytes : 1);
+    int splits = env > 0 ? env : (3 * resident + 2 * tiles_n) / (4 * tiles_n);
     if (splits > slabs / 4) splits = slabs / 4;
     if (splits < 1) splits = 1;
     if (splits > 64) splits = 64;
@@ -171,7 +174,7 @@ int mi_gemm_config_grid(int config, int M, int N, int K) {
     if (e.kind == mi::KIND_SKINNY) {
         if (M > e.BM || K % 64 != 0) return 0;
         const int tiles_n = (N + e.BN - 1) / e.BN;
-        return tiles_n * choose_splits(tiles_n, K, compute_units());
+        return tiles_n * choose_splits(tiles_n, K, compute_units(), e.lds_bytes);
     }
     return ((M + e.BM - 1) / e.BM) * ((N + e.BN - 1) / e.BN);
 }
@@ -234,7 +237,7 @@ int mi_gemm_ex(int config, int dtype, int M, int N, int K, const void* A, const 
                         "config %s needs M <= %d, N %% 4 == 0, K %% 64 == 0 and 16-byte aligned operands",
                         e.name, e.BM);
         const int tiles_n = (N + e.BN - 1) / e.BN;
-        args.splits = choose_splits(tiles_n, K, compute_units());   // <= K / 64: no empty split
+        args.splits = choose_splits(tiles_n, K, compute_units(), e.lds_bytes);   // <= K / 64: no empty split
         args.k_per_split = ((K / 64 + args.splits - 1) / args.splits) * 64;
         if (args.splits > 1) {
             hipError_t we = ensure_workspace((size_t)args.splits * M * N * sizeof(float), &args.ws);

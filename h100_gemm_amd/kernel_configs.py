@@ -192,3 +192,9 @@ TUNED_SHAPES = {
     (8192, 28672, 8192): "t256x256_w2x2_s1_g4_o1_d1_e1_x2x4",
 }
 assert all(n in {config_name(c) for c in CONFIGS} for n in TUNED_SHAPES.values())
+
+# Automatic choice for decode shapes (the kernels' preconditions permitting): (largest M,
+# config name), first match wins.  Up to M = 32 the single-pass kernel; above, the split-K
+# kernel measured ahead of it (M = 64: 30 us against 33 us).
+DECODE_LADDER = [(16, "s16x32_n5"), (32, "s32x32_n4"), (64, "k64x128_n6"), (128, "k128x128_n5")]
+assert all(n in {config_name(c) for c in CONFIGS} for _, n in DECODE_LADDER)
