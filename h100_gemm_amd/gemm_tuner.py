@@ -71,9 +71,9 @@ class GemmTuner:
 
         # Define parameter search space
         self.param_space = {
-            'KIND': ['ring', 'tile'],
+            'KIND': ['mfma16', 'ring', 'ring16', 'tile'],
             'BM': [128, 256],
-            'BN': [128, 256],
+            'BN': [128, 192, 256],
             'WM': [2, 4],
             'WN': [2, 4],
             'NS': [4],
@@ -154,10 +154,10 @@ class GemmTuner:
     def is_valid_configuration(self, params: Dict[str, int]) -> bool:
         """Check if a parameter configuration is valid"""
         c = dict(params, OCC=1)
-        if c['KIND'] == 'ring' and (c.get('SWZ', 1) != 1 or c.get('DTL', 1) != 1 or c.get('EPI', 1) != 1):
-            return False            # the ring kernel has one load path and one epilogue
-        if c['KIND'] == 'tile' and c.get('NS', 4) != self.param_space['NS'][0]:
-            return False            # NS is meaningless for the two-stage kernel: keep one copy
+        if c['KIND'] != 'tile' and (c.get('SWZ', 1) != 1 or c.get('DTL', 1) != 1 or c.get('EPI', 1) != 1):
+            return False            # only the two-stage kernel has several load paths and epilogues
+        if c['KIND'] in ('tile', 'mfma16') and c.get('NS', 4) != self.param_space['NS'][0]:
+            return False            # NS is meaningless for the two-stage kernels: keep one copy
         try:
             return kc.is_valid_config(c)
         except KeyError:

@@ -60,6 +60,11 @@ def lds_bytes(c: dict) -> int:
 
 def is_valid_config(c: dict) -> bool:
     """Static rules of the kernels (mirrored as static_asserts in csrc/)."""
+    if c["KIND"] in ("ring", "mfma16", "ring16") and not c.get("_twin_checked"):
+        # ragged shapes run the predicated two-stage kernel of the same tile and wave grid
+        twin = dict(KIND="tile", BM=c["BM"], BN=c["BN"], WM=c["WM"], WN=c["WN"], SWZ=1,
+                    GROUP=c["GROUP"], OCC=1, DTL=0, EPI=1)
+        return is_valid_config(twin) and is_valid_config(dict(c, _twin_checked=True))
     if c["KIND"] == "tile" and (c.get("EWM", c["WM"]), c.get("EWN", c["WN"])) != (c["WM"], c["WN"]):
         twin = dict(c, WM=c["EWM"], WN=c["EWN"], DTL=0)
         del twin["EWM"], twin["EWN"]
