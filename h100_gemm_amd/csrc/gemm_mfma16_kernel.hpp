@@ -47,10 +47,11 @@ struct Mfma16Config {
     static constexpr int LDS_BYTES = 2 * (A_STAGE + B_STAGE);
     static constexpr int WAVES_PER_EU = NT / 256;
     static constexpr int NMMA = MI * NI, NFR = MI + NI;
-    static_assert(NT == 512, "two waves per SIMD");
+    static_assert(NT == 256 || NT == 512, "one or two waves per SIMD");
     static_assert(TM % 16 == 0 && TN % 16 == 0, "wave tile must be a multiple of 16x16");
     static_assert(BM % RPP == 0 && BN % RPP == 0 && RPP % 16 == 0, "tile rows divide over the threads");
-    static_assert(NFR + 2 * (LA + LB) <= NMMA, "reads and loads each get an MFMA slot");
+    static constexpr int DSP = (NMMA - NFR) / (LA + LB);   // MFMA slots between two load instructions
+    static_assert(DSP >= 1, "reads and loads each get an MFMA slot");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
     static_assert(BM * BN * 2 <= LDS_BYTES, "the epilogue stages the C tile in the stage buffers");
 };
@@ -168,7 +169,7 @@ gemm_mfma16_kernel(const GemmArgs p) {
 #pragma unroll
     for (int r = 0; r < NFR; ++r) read_one(0, 0, 0, r);
 
-    // load instruction slots of slice 1: every other MFMA after the fragment reads
+    // load instruction slots of slice 1: spread evenly over the MFMAs that follow the fragment reads
     auto kstep = [&](int kt, auto cur_c, auto has1_c, auto has2_c) __attribute__((always_inline)) {
         constexpr int cur = decltype(cur_c)::value;
         constexpr int nxt = cur ^ 1;
@@ -193,7 +194,7 @@ gemm_mfma16_kernel(const GemmArgs p) {
             }
             if constexpr (has2) {
                 const int d = idx - NFR;
-                if (d >= 0 && (d & 1) == 0 && d / 2 < LA + LB) dma_one(kt + 2, cur, d / 2);
+                if (d >= 0 && d % Cfg::DSP == 0 && d / Cfg::DSP < LA + LB) dma_one(kt + 2, cur, d / Cfg::DSP);
             }
 
             __builtin_amdgcn_sched_barrier(0);
@@ -266,7 +267,9 @@ gemm_mfma16_kernel(const GemmArgs p) {
 // ---------------------------------------------------------------------------------------
 // Ring variant: K slab = one 32-deep MFMA slice (64-byte LDS rows, chunks stored at
 // chunk ^ ((row >> 2) & 3)), NS stages, loads issued NS slabs ahead and dealt out one per
-// few MFMAs, `vmcnt((NS-2)*L)` waits (never on the youngest loads), one barrier per slab.
+// few MFMAs (spread evenly over the slots that follow the fragment reads, so that the four
+// or eight waves of a CU do not queue up at the texture addresser), `vmcnt((NS-2)*L)` waits
+// (never on the youngest loads), one barrier per slab.
 // A slab has NS-1 steps (~3000 cycles at NS = 4) to land instead of ~1.
 template <int BM_, int BN_, int WM_, int WN_, int NS_, int GROUP_, int DT_>
 struct Ring16Config {
@@ -282,10 +285,11 @@ struct Ring16Config {
     static constexpr int LDS_BYTES = NS * STAGE;
     static constexpr int WAVES_PER_EU = NT / 256;
     static constexpr int NMMA = MI * NI, NFR = MI + NI;
-    static_assert(NT == 512, "two waves per SIMD");
+    static constexpr int DSP = (NMMA - NFR) / L;         // MFMA slots between two load instructions
+    static_assert(NT == 256 || NT == 512, "one or two waves per SIMD");
     static_assert(TM % 16 == 0 && TN % 16 == 0, "wave tile must be a multiple of 16x16");
     static_assert(BM % RPP == 0 && BN % RPP == 0, "tile rows divide over the waves");
-    static_assert(NFR + 2 * L <= NMMA, "reads and loads each get an MFMA slot");
+    static_assert(DSP >= 1, "reads and loads each get an MFMA slot");
     static_assert(NS >= 3 && NS <= 5 && (NS - 1) * L <= 63, "vmcnt is a 6-bit counter");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
     static_assert(BM * BN * 2 <= LDS_BYTES, "the epilogue stages the C tile in the ring");
@@ -403,7 +407,7 @@ gemm_ring16_kernel(const GemmArgs p) {
             mma_one(buf, idx);
             if (idx < NFR) read_one(sn, buf ^ 1, idx);
             const int d = idx - NFR;
-            if (d >= 0 && (d & 1) == 0 && d / 2 < L) dma_one(t + NS, s, d / 2);
+            if (d >= 0 && d % Cfg::DSP == 0 && d / Cfg::DSP < L) dma_one(t + NS, s, d / Cfg::DSP);
             __builtin_amdgcn_sched_barrier(0);
         }
     };

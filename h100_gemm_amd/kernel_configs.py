@@ -13,7 +13,7 @@ template takes (matmul_h100.cu.jinja:9-14) -- re-cast for CDNA4:
     KIND     "tile" (two-stage kernel above), "ring" (NS-deep LDS ring, K step 32, aligned
              shapes; ragged shapes take the predicated tile kernel of the same tile),
              "mfma16" / "ring16" (the same two pipelines on the 16x16x32 MFMA with eight
-             waves, csrc/gemm_mfma16_kernel.hpp), or "skinny" (split-K streaming kernel for
+             or four waves, csrc/gemm_mfma16_kernel.hpp), or "skinny" (split-K streaming kernel for
              M <= BM, decode shapes)
     EPI      1: C tile transposed through LDS and written 16 bytes per lane, 0: 8-byte stores
     EWM, EWN (optional) wave grid of the predicated twin when it differs from WM, WN (the
@@ -30,7 +30,10 @@ def config_name(c: dict) -> str:
     if c["KIND"] == "ring":
         return f"r{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_n{c['NS']}_g{c['GROUP']}"
     if c["KIND"] == "mfma16":
-        return f"m{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_g{c['GROUP']}"
+        name = f"m{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_g{c['GROUP']}"
+        if (c.get("EWM", c["WM"]), c.get("EWN", c["WN"])) != (c["WM"], c["WN"]):
+            name += f"_x{c['EWM']}x{c['EWN']}"
+        return name
     if c["KIND"] == "ring16":
         return f"q{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_n{c['NS']}_g{c['GROUP']}"
     if c["KIND"] == "skinny":
@@ -62,7 +65,7 @@ def is_valid_config(c: dict) -> bool:
     """Static rules of the kernels (mirrored as static_asserts in csrc/)."""
     if c["KIND"] in ("ring", "mfma16", "ring16") and not c.get("_twin_checked"):
         # ragged shapes run the predicated two-stage kernel of the same tile and wave grid
-        twin = dict(KIND="tile", BM=c["BM"], BN=c["BN"], WM=c["WM"], WN=c["WN"], SWZ=1,
+        twin = dict(KIND="tile", BM=c["BM"], BN=c["BN"], WM=c.get("EWM", c["WM"]), WN=c.get("EWN", c["WN"]), SWZ=1,
                     GROUP=c["GROUP"], OCC=1, DTL=0, EPI=1)
         return is_valid_config(twin) and is_valid_config(dict(c, _twin_checked=True))
     if c["KIND"] == "tile" and (c.get("EWM", c["WM"]), c.get("EWN", c["WN"])) != (c["WM"], c["WN"]):
@@ -93,11 +96,12 @@ def is_valid_config(c: dict) -> bool:
         return False
     waves_per_simd = max(nt // 256, 1) * occ
     if c["KIND"] in ("mfma16", "ring16"):
-        # 16x16x32 MFMA kernels: eight waves, 4 accumulator registers per 16x16 tile
-        if nt != 512 or c["BM"] * c["BN"] * 2 > lds_bytes(c):
+        # 16x16x32 MFMA kernels: 4 accumulator registers per 16x16 tile; the two-stage kernel
+        # runs with four or eight waves, the ring kernel with eight
+        if nt not in (256, 512) or c["BM"] * c["BN"] * 2 > lds_bytes(c):
             return False
         mi16, ni16 = 2 * mi, 2 * ni
-        rpp = 64 if c["KIND"] == "mfma16" else 128
+        rpp = nt // 8 if c["KIND"] == "mfma16" else nt // 4
         if c["BM"] % rpp or c["BN"] % rpp:
             return False
         l = c["BM"] // rpp + c["BN"] // rpp
@@ -106,9 +110,9 @@ def is_valid_config(c: dict) -> bool:
         tn = c["BN"] // c["WN"]
         if tn & (tn - 1) or tn < 32:          # the C staging swizzle needs a power-of-two row
             return False
-        if mi16 + ni16 + 2 * l > mi16 * ni16:
+        if mi16 + ni16 + l > mi16 * ni16:
             return False
-        return mi16 * ni16 * 4 + 2 * (mi16 + ni16) * 4 + 24 <= 256
+        return mi16 * ni16 * 4 + 2 * (mi16 + ni16) * 4 + 24 <= 512 // waves_per_simd
     if c["KIND"] == "ring":
         rpp = (nt // 64) * 16
         if c["BM"] % rpp or c["BN"] % rpp or c["NS"] != 4:
@@ -141,8 +145,10 @@ def _r(BM, BN, WM, WN, NS=4, GROUP=8):
     return dict(KIND="ring", BM=BM, BN=BN, WM=WM, WN=WN, NS=NS, GROUP=GROUP)
 
 
-def _m(BM, BN, WM, WN, GROUP=4, EFF=None):
+def _m(BM, BN, WM, WN, GROUP=4, EFF=None, EW=None):
     c = dict(KIND="mfma16", BM=BM, BN=BN, WM=WM, WN=WN, GROUP=GROUP)
+    if EW is not None:
+        c["EWM"], c["EWN"] = EW
     if EFF is not None:
         c["EFF"] = EFF
     return c
@@ -164,7 +170,7 @@ CONFIGS = [
     _c(256, 256, 2, 2, SWZ=1, GROUP=8),
     _c(256, 256, 2, 2, SWZ=1, GROUP=8, DTL=1),
     _c(256, 256, 2, 2, SWZ=1, GROUP=8, DTL=1, EPI=1),
-    _c(256, 256, 2, 2, SWZ=1, GROUP=4, DTL=1, EPI=1, EFF=0.96, EW=(2, 4)),
+    _c(256, 256, 2, 2, SWZ=1, GROUP=4, DTL=1, EPI=1, EFF=0.9, EW=(2, 4)),
     _c(256, 256, 2, 4, SWZ=1, GROUP=8, DTL=1, EPI=1),
     _c(256, 192, 2, 2, SWZ=1, GROUP=4, DTL=1, EPI=1),
     _c(256, 192, 2, 2, SWZ=1, GROUP=4, DTL=1, EPI=1, EFF=0.89, EW=(4, 2)),
@@ -175,9 +181,11 @@ CONFIGS = [
     _c(128, 128, 2, 2, SWZ=1, GROUP=8, OCC=2, DTL=1, EPI=1, EFF=0.83),
     _r(256, 256, 2, 2),
     _r(256, 256, 2, 4),
-    _m(256, 256, 4, 2, EFF=1.0),
+    _m(256, 256, 2, 2, EFF=1.0, EW=(2, 4)),
+    _m(256, 256, 4, 2),
     _m(256, 256, 2, 4),
     _q(256, 256, 4, 2),
+    _q(256, 256, 2, 2),
     _s(16, 5),
     _s(32, 4),
     _s(64, 3),
@@ -189,13 +197,10 @@ CONFIGS = [
 assert all(is_valid_config(c) for c in CONFIGS), [config_name(c) for c in CONFIGS if not is_valid_config(c)]
 assert len({config_name(c) for c in CONFIGS}) == len(CONFIGS)
 
-# Exact shapes with a tuned choice (config name), consulted before the cost model.  Across
-# shapes the eight-wave 16x16x32-MFMA kernel is the steadier 256x256 kernel (5-11 % ahead at
-# 4096^3, K = 12288 .. 28672), the four-wave 32x32x16 kernel is 1-3 % ahead at these two.
-TUNED_SHAPES = {
-    (8192, 8192, 8192): "t256x256_w2x2_s1_g4_o1_d1_e1_x2x4",
-    (8192, 28672, 8192): "t256x256_w2x2_s1_g4_o1_d1_e1_x2x4",
-}
+# Exact shapes with a tuned choice (config name), consulted before the cost model.  Empty at
+# present: the four-wave 16x16x32-MFMA kernel is ahead at every aligned shape measured
+# (8192^3, both MLP shapes, 4096^3, K = 12288 .. 28672).
+TUNED_SHAPES = {}
 assert all(n in {config_name(c) for c in CONFIGS} for n in TUNED_SHAPES.values())
 
 # Automatic choice for decode shapes (the kernels' preconditions permitting): (largest M,

@@ -109,6 +109,7 @@ def test_config_table(mi):
     # exact shapes with a tuned entry take it; everything else goes through the cost model
     for (M, N, K), name in kc.TUNED_SHAPES.items():
         assert mi.config_name(mi.select_config(M, N, K)) == name
+    assert kc.CONFIGS[mi.select_config(8192, 8192, 8192)]["KIND"] == "mfma16"
     assert kc.CONFIGS[mi.select_config(4096, 4096, 4096)]["KIND"] == "mfma16"
     # wave quantisation: 256 CUs; 8192^2 fills four rounds of 256x256 tiles, 4095x6143 fills
     # two rounds of 256x192 tiles exactly (256x256 would leave half of the second round
