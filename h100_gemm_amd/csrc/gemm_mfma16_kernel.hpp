@@ -34,10 +34,11 @@ namespace mi {
 
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
-template <int BM_, int BN_, int WM_, int WN_, int GROUP_, int DT_>
+template <int BM_, int BN_, int WM_, int WN_, int GROUP_, int DT_, int DRAIN_ = 0>
 struct Mfma16Config {
     static constexpr int BM = BM_, BN = BN_, BK = 64;
     static constexpr int WM = WM_, WN = WN_, GROUP = GROUP_, DT = DT_;
+    static constexpr bool DRAIN = DRAIN_ != 0;
     static constexpr int NT = WM * WN * 64, NW = WM * WN;
     static constexpr int TM = BM / WM, TN = BN / WN;
     static constexpr int MI = TM / 16, NI = TN / 16;
@@ -52,6 +53,14 @@ struct Mfma16Config {
     static_assert(BM % RPP == 0 && BN % RPP == 0 && RPP % 16 == 0, "tile rows divide over the threads");
     static constexpr int DSP = (NMMA - NFR) / (LA + LB);   // MFMA slots between two load instructions
     static_assert(DSP >= 1, "reads and loads each get an MFMA slot");
+    // DRAIN > 0: a second barrier early in slice 0 (slot SA = NFR + 4*DRAIN, once every wave has fetched the
+    // slice-1 fragments) frees the current stage, so the loads of the slab after next are
+    // dealt out over the rest of slice 0 and all of slice 1 (slots SA+1 + d*DSPD of the
+    // step) and have a whole K step to land; D0 of them are issued before the mid-step wait.
+    static constexpr int SA = NFR + 4 * DRAIN_;
+    static constexpr int DSPD = (2 * NMMA - 5 - SA) / (LA + LB);
+    static constexpr int D0 = DSPD > 0 ? (NMMA - SA - 1 + DSPD - 1) / DSPD : 0;
+    static_assert(!DRAIN || (DSPD >= 1 && SA + 1 < NMMA && D0 <= LA + LB), "drain schedule");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
     static_assert(BM * BN * 2 <= LDS_BYTES, "the epilogue stages the C tile in the stage buffers");
 };
@@ -115,17 +124,23 @@ gemm_mfma16_kernel(const GemmArgs p) {
     const uint32_t passB = (uint32_t)(RPP * p.ldb) * 2u;
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
     const uint32_t dlds = lds_base + (uint32_t)wave * 1024u;
-    auto dma = [&](const __amdgpu_buffer_rsrc_t& rsrc, uint32_t voff, uint32_t dst) __attribute__((always_inline)) {
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-                     :: "s"(dst), "v"(voff), "s"(rsrc) : "memory");
+    // per-lane byte offsets of every load instruction of a slab, kept in registers; the K
+    // offset of the slab goes in the instruction's scalar offset, so a load costs no VALU work
+    uint32_t voffs[LA + LB];
+#pragma unroll
+    for (int d = 0; d < LA; ++d) voffs[d] = dvoffA + d * passA;
+#pragma unroll
+    for (int d = 0; d < LB; ++d) voffs[LA + d] = dvoffB + d * passB;
+    auto dma = [](__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff, uint32_t dst) __attribute__((always_inline)) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                     :: "s"(dst), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
     };
     auto dma_one = [&](int kt, int stage, int d) __attribute__((always_inline)) {
         const uint32_t kb = (uint32_t)kt * (BK * 2);
         if (d < LA)
-            dma(rsrcA, dvoffA + kb + d * passA, dlds + stage * A_STAGE + d * (RPP * 128));
+            dma(rsrcA, voffs[d], kb, dlds + stage * A_STAGE + d * (RPP * 128));
         else
-            dma(rsrcB, dvoffB + kb + (d - LA) * passB,
-                dlds + 2 * A_STAGE + stage * B_STAGE + (d - LA) * (RPP * 128));
+            dma(rsrcB, voffs[d], kb, dlds + 2 * A_STAGE + stage * B_STAGE + (d - LA) * (RPP * 128));
     };
 
     // fragment reads: lane holds row (lane & 15), k chunk 4*ks + (lane >> 4) of the slab
@@ -175,15 +190,36 @@ gemm_mfma16_kernel(const GemmArgs p) {
         constexpr int nxt = cur ^ 1;
         constexpr bool has1 = decltype(has1_c)::value;
         constexpr bool has2 = decltype(has2_c)::value;
+        // load d of slab kt+2 goes out at slot g of the step (slice 0: g < NMMA)
+        auto dma_slot = [&](int g) __attribute__((always_inline)) {
+            if constexpr (has2) {
+                if constexpr (Cfg::DRAIN) {
+                    const int d = g - (Cfg::SA + 1);
+                    if (d >= 0 && d % Cfg::DSPD == 0 && d / Cfg::DSPD < LA + LB) dma_one(kt + 2, cur, d / Cfg::DSPD);
+                } else {
+                    const int d = g - NMMA - NFR;
+                    if (d >= 0 && d % Cfg::DSP == 0 && d / Cfg::DSP < LA + LB) dma_one(kt + 2, cur, d / Cfg::DSP);
+                }
+            }
+        };
 #pragma unroll
         for (int idx = 0; idx < NMMA; ++idx) {
             mma_one(0, idx);
             if (idx < NFR) read_one(cur, 1, 1, idx);
+            if constexpr (Cfg::DRAIN && has2) {
+                // every wave holds its slice-1 fragments: stage `cur` may be overwritten
+                if (idx == Cfg::SA) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            }
+            dma_slot(idx);
             __builtin_amdgcn_sched_barrier(0);
         }
         if constexpr (has1) {
             if constexpr (TRACE) tr_t0 = tr_now();
-            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            // slab kt+1 has landed (the D0 younger loads of slab kt+2 may still be in flight)
+            if constexpr (Cfg::DRAIN && has2)
+                asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" :: "n"(Cfg::D0) : "memory");
+            else
+                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
             if constexpr (TRACE) { tr_wait += tr_now() - tr_t0; ++tr_cnt; }
         }
 #pragma unroll
@@ -192,11 +228,7 @@ gemm_mfma16_kernel(const GemmArgs p) {
             if constexpr (has1) {
                 if (idx < NFR) read_one(nxt, 0, 0, idx);
             }
-            if constexpr (has2) {
-                const int d = idx - NFR;
-                if (d >= 0 && d % Cfg::DSP == 0 && d / Cfg::DSP < LA + LB) dma_one(kt + 2, cur, d / Cfg::DSP);
-            }
-
+            dma_slot(NMMA + idx);
             __builtin_amdgcn_sched_barrier(0);
         }
     };

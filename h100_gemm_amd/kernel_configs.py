@@ -16,6 +16,9 @@ template takes (matmul_h100.cu.jinja:9-14) -- re-cast for CDNA4:
              or four waves, csrc/gemm_mfma16_kernel.hpp), or "skinny" (split-K streaming kernel for
              M <= BM, decode shapes)
     EPI      1: C tile transposed through LDS and written 16 bytes per lane, 0: 8-byte stores
+    DRAIN    (mfma16, optional) d > 0: a second barrier early in each K step (4*d MFMAs after the
+             fragment reads) frees the current LDS stage, so the next loads are spread over most
+             of the step instead of its second half
     EWM, EWN (optional) wave grid of the predicated twin when it differs from WM, WN (the
              register-staged predicated kernel runs best with eight waves)
     EFF      (optional) per-CU throughput relative to the 256x256 tile, measured at 8192^3;
@@ -31,6 +34,8 @@ def config_name(c: dict) -> str:
         return f"r{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_n{c['NS']}_g{c['GROUP']}"
     if c["KIND"] == "mfma16":
         name = f"m{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_g{c['GROUP']}"
+        if c.get("DRAIN", 0):
+            name += "_b2"
         if (c.get("EWM", c["WM"]), c.get("EWN", c["WN"])) != (c["WM"], c["WN"]):
             name += f"_x{c['EWM']}x{c['EWN']}"
         return name
@@ -145,8 +150,10 @@ def _r(BM, BN, WM, WN, NS=4, GROUP=8):
     return dict(KIND="ring", BM=BM, BN=BN, WM=WM, WN=WN, NS=NS, GROUP=GROUP)
 
 
-def _m(BM, BN, WM, WN, GROUP=4, EFF=None, EW=None):
+def _m(BM, BN, WM, WN, GROUP=4, EFF=None, EW=None, DRAIN=0):
     c = dict(KIND="mfma16", BM=BM, BN=BN, WM=WM, WN=WN, GROUP=GROUP)
+    if DRAIN:
+        c["DRAIN"] = DRAIN
     if EW is not None:
         c["EWM"], c["EWN"] = EW
     if EFF is not None:
@@ -181,8 +188,10 @@ CONFIGS = [
     _c(128, 128, 2, 2, SWZ=1, GROUP=8, OCC=2, DTL=1, EPI=1, EFF=0.83),
     _r(256, 256, 2, 2),
     _r(256, 256, 2, 4),
-    _m(256, 256, 2, 2, EFF=1.0, EW=(2, 4)),
+    _m(256, 256, 2, 2, EW=(2, 4)),
+    _m(256, 256, 2, 2, DRAIN=3, EFF=1.0, EW=(2, 4)),
     _m(256, 256, 4, 2),
+    _m(256, 256, 4, 2, DRAIN=3),
     _m(256, 256, 2, 4),
     _q(256, 256, 4, 2),
     _q(256, 256, 2, 2),
