@@ -34,11 +34,12 @@ namespace mi {
 
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
-template <int BM_, int BN_, int WM_, int WN_, int GROUP_, int DT_, int DRAIN_ = 0>
+template <int BM_, int BN_, int WM_, int WN_, int GROUP_, int DT_, int DRAIN_ = 0, bool EDGE_ = false>
 struct Mfma16Config {
     static constexpr int BM = BM_, BN = BN_, BK = 64;
     static constexpr int WM = WM_, WN = WN_, GROUP = GROUP_, DT = DT_;
     static constexpr bool DRAIN = DRAIN_ != 0;
+    static constexpr bool EDGE = EDGE_;                  // predicated variant: any M, N, K, any alignment
     static constexpr int NT = WM * WN * 64, NW = WM * WN;
     static constexpr int TM = BM / WM, TN = BN / WN;
     static constexpr int MI = TM / 16, NI = TN / 16;
@@ -102,13 +103,20 @@ gemm_mfma16_kernel(const GemmArgs p) {
     int tm, tn;
     tile_of_block<Cfg::GROUP>(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, tm, tn);
     const int row0 = tm * BM, col0 = tn * BN;
-    const int K = p.K;
-    const int KT = K / BK;                               // even (host checks K % 128 == 0)
+    constexpr bool EDGE = Cfg::EDGE;
+    const int M = p.M, N = p.N, K = p.K;
+    // K steps: an even number.  The aligned variant is only launched with K % 128 == 0; the
+    // predicated one rounds up and the surplus (part of a) slab is zeroed in LDS.
+    const int KT = EDGE ? ((K + 2 * BK - 1) / (2 * BK)) * 2 : K / BK;
 
+    // Descriptors end exactly at the last element of the tile's last valid row: nothing past
+    // the end of a matrix is ever touched, and rows past M / N read as zeros.
+    const int rowsA = (M - row0) < BM ? (M - row0) : BM;
+    const int rowsB = (N - col0) < BN ? (N - col0) : BN;
     const unsigned char* Ab = (const unsigned char*)p.A + (size_t)row0 * p.lda * 2;
     const unsigned char* Bb = (const unsigned char*)p.B + (size_t)col0 * p.ldb * 2;
-    const uint32_t bytesA = (uint32_t)((BM - 1) * p.lda + K) * 2u;
-    const uint32_t bytesB = (uint32_t)((BN - 1) * p.ldb + K) * 2u;
+    const uint32_t bytesA = (uint32_t)((rowsA - 1) * p.lda + K) * 2u;
+    const uint32_t bytesB = (uint32_t)((rowsB - 1) * p.ldb + K) * 2u;
     const __amdgpu_buffer_rsrc_t rsrcA = __builtin_amdgcn_make_buffer_rsrc((void*)Ab, 0, (int)bytesA, 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrcB = __builtin_amdgcn_make_buffer_rsrc((void*)Bb, 0, (int)bytesB, 0x00020000);
 
@@ -141,6 +149,49 @@ gemm_mfma16_kernel(const GemmArgs p) {
             dma(rsrcA, voffs[d], kb, dlds + stage * A_STAGE + d * (RPP * 128));
         else
             dma(rsrcB, voffs[d], kb, dlds + 2 * A_STAGE + stage * B_STAGE + (d - LA) * (RPP * 128));
+    };
+
+    // K tail (predicated variant).  A direct-to-LDS load of the chunk at k..k+7 of a row runs
+    // into the next row of the matrix when k+7 >= K (or returns zeros past the descriptor), so
+    // once its own loads of a slab have landed, each lane zeroes what it fetched at k >= K, in
+    // LDS, before the barrier that publishes the slab.  The range check works on whole
+    // dwords: the dword holding the last element (k = K-1) of the tile's last row is dropped
+    // whenever its other half lies past the descriptor's end, so that one element per operand
+    // is fetched by a 2-byte load up front (tailA / tailB) and put back here.  This lane's
+    // logical chunk is the same for all its loads (the swizzle repeats every 16 rows).
+    uint32_t tailA = 0, tailB = 0;
+    if constexpr (EDGE) {
+        tailA = __builtin_amdgcn_readfirstlane(__builtin_amdgcn_raw_buffer_load_b16(rsrcA, bytesA - 2u, 0, 0));
+        tailB = __builtin_amdgcn_readfirstlane(__builtin_amdgcn_raw_buffer_load_b16(rsrcB, bytesB - 2u, 0, 0));
+    }
+    auto fix_tail = [&](int kt, int stage) __attribute__((always_inline)) {
+        const int nvalid = K - (kt * BK + dchunk * 8);   // elements of this lane's chunk that lie inside K
+        if (nvalid >= 8) return;
+        const int kl = nvalid - 1;                       // where k = K-1 sits in this chunk
+        const bool mine = kl >= 0;
+        uint32_t m[4];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            const int n = nvalid - 2 * d;
+            m[d] = n >= 2 ? 0xffffffffu : (n == 1 ? 0x0000ffffu : 0u);
+        }
+        // rolled loops: this runs for the last two slabs only and must not cost registers
+        auto fix_rows = [&](unsigned char* ptr, int passes, int last_row, uint32_t e) __attribute__((always_inline)) {
+#pragma clang loop unroll(disable)
+            for (int d = 0; d < passes; ++d, ptr += RPP * 128) {
+                u32x4_t v = *(const u32x4_t*)ptr;
+                const bool hit = mine && d * RPP + drow == last_row;
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    const uint32_t old = v[w];
+                    const uint32_t pv = (kl & 1) ? ((old & 0x0000ffffu) | (e << 16)) : ((old & 0xffff0000u) | e);
+                    v[w] = ((hit && (kl >> 1) == w) ? pv : old) & m[w];
+                }
+                *(u32x4_t*)ptr = v;
+            }
+        };
+        fix_rows(lds + stage * A_STAGE + wave * 1024 + lane * 16, LA, rowsA - 1, tailA);
+        fix_rows(lds + 2 * A_STAGE + stage * B_STAGE + wave * 1024 + lane * 16, LB, rowsB - 1, tailB);
     };
 
     // fragment reads: lane holds row (lane & 15), k chunk 4*ks + (lane >> 4) of the slab
@@ -180,16 +231,23 @@ gemm_mfma16_kernel(const GemmArgs p) {
     for (int d = 0; d < LA + LB; ++d) dma_one(0, 0, d);
 #pragma unroll
     for (int d = 0; d < LA + LB; ++d) dma_one(1, 1, d);
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"(LA + LB) : "memory");    // slab 0 is in
+    if constexpr (EDGE) {
+        asm volatile("s_waitcnt vmcnt(%0)" :: "n"(LA + LB) : "memory");            // own loads of slab 0 are in
+        if (BK > K) fix_tail(0, 0);
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    } else {
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"(LA + LB) : "memory");    // slab 0 is in
+    }
 #pragma unroll
     for (int r = 0; r < NFR; ++r) read_one(0, 0, 0, r);
 
     // load instruction slots of slice 1: spread evenly over the MFMAs that follow the fragment reads
-    auto kstep = [&](int kt, auto cur_c, auto has1_c, auto has2_c) __attribute__((always_inline)) {
+    auto kstep = [&](int kt, auto cur_c, auto has1_c, auto has2_c, auto fix_c) __attribute__((always_inline)) {
         constexpr int cur = decltype(cur_c)::value;
         constexpr int nxt = cur ^ 1;
         constexpr bool has1 = decltype(has1_c)::value;
         constexpr bool has2 = decltype(has2_c)::value;
+        constexpr bool fix = decltype(fix_c)::value;       // slab kt+1 may cross K (predicated variant)
         // load d of slab kt+2 goes out at slot g of the step (slice 0: g < NMMA)
         auto dma_slot = [&](int g) __attribute__((always_inline)) {
             if constexpr (has2) {
@@ -216,10 +274,18 @@ gemm_mfma16_kernel(const GemmArgs p) {
         if constexpr (has1) {
             if constexpr (TRACE) tr_t0 = tr_now();
             // slab kt+1 has landed (the D0 younger loads of slab kt+2 may still be in flight)
-            if constexpr (Cfg::DRAIN && has2)
+            if constexpr (fix) {
+                if constexpr (Cfg::DRAIN && has2)
+                    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" :: "n"(Cfg::D0) : "memory");
+                else
+                    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                fix_tail(kt + 1, nxt);
+                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            } else if constexpr (Cfg::DRAIN && has2) {
                 asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" :: "n"(Cfg::D0) : "memory");
-            else
+            } else {
                 asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            }
             if constexpr (TRACE) { tr_wait += tr_now() - tr_t0; ++tr_cnt; }
         }
 #pragma unroll
@@ -237,12 +303,28 @@ gemm_mfma16_kernel(const GemmArgs p) {
     using S0 = std::integral_constant<int, 0>;
     using S1 = std::integral_constant<int, 1>;
     int kt = 0;
-    for (; kt + 2 < KT; kt += 2) {
-        kstep(kt, S0{}, T{}, T{});
-        kstep(kt + 1, S1{}, T{}, T{});
+    if constexpr (!EDGE) {
+        for (; kt + 2 < KT; kt += 2) {
+            kstep(kt, S0{}, T{}, T{}, F{});
+            kstep(kt + 1, S1{}, T{}, T{}, F{});
+        }
+        kstep(kt, S0{}, T{}, F{}, F{});
+        kstep(kt + 1, S1{}, F{}, F{}, F{});
+    } else {
+        // Only the last two slabs can cross K (KT is rounded up to even); the steps that
+        // publish them are peeled off so that the steady-state loop carries no fix-up code.
+        if (KT >= 4) {
+            for (; kt + 4 < KT; kt += 2) {
+                kstep(kt, S0{}, T{}, T{}, F{});
+                kstep(kt + 1, S1{}, T{}, T{}, F{});
+            }
+            kstep(kt, S0{}, T{}, T{}, F{});
+            kstep(kt + 1, S1{}, T{}, T{}, T{});
+            kt += 2;
+        }
+        kstep(kt, S0{}, T{}, F{}, T{});
+        kstep(kt + 1, S1{}, F{}, F{}, F{});
     }
-    kstep(kt, S0{}, T{}, F{});
-    kstep(kt + 1, S1{}, F{}, F{});
 
     long long tr_store = 0;
     if constexpr (TRACE) {
@@ -252,11 +334,19 @@ gemm_mfma16_kernel(const GemmArgs p) {
     // ---- epilogue: C tile -> storage type -> per-wave LDS staging -> 16-byte row stores ----
     // acc[i][j][e] of lane l is C[m][n], m = i*16 + (l & 15), n = j*16 + 4*(l >> 4) + e
     unsigned char* Cb = (unsigned char*)p.C + (size_t)row0 * p.ldc * 2;
-    const uint32_t bytesC = (uint32_t)(BM * p.ldc) * 2u;
+    const uint32_t bytesC = (uint32_t)(rowsA * p.ldc) * 2u;
     const __amdgpu_buffer_rsrc_t rsrcC = __builtin_amdgcn_make_buffer_rsrc((void*)Cb, 0, (int)bytesC, 0x00020000);
     {
+        // The predicated variant masks rows past M, stores 16 bytes at any 2-byte boundary
+        // (odd N) and splits only the chunk that straddles N into 2-byte stores.
         constexpr int CPR = TN / 8;                 // 16-byte chunks per row of the wave tile
-        constexpr int RPI = 64 / CPR;               // rows per read/store instruction
+        constexpr bool POW2 = (CPR & (CPR - 1)) == 0;
+        static_assert(CPR % 2 == 0 && (TM * CPR) % 64 == 0, "C staging layout");
+        // rows of a power-of-two width are spread over the banks by the row number, 192-byte
+        // rows (4 rows = 3 bank rounds) by row / 4
+        auto cswz = [](int row) __attribute__((always_inline)) {
+            return POW2 ? (row & (CPR - 1)) : ((row >> 2) & 3);
+        };
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");   // all waves done with the last stage
         unsigned char* stg = lds + wave * (TM * TN * 2);
 #pragma unroll
@@ -264,7 +354,7 @@ gemm_mfma16_kernel(const GemmArgs p) {
             const int row = i * 16 + l16;
 #pragma unroll
             for (int j = 0; j < NI; ++j) {
-                const int chunk = (j * 2 + (q >> 1)) ^ (row & (CPR - 1));
+                const int chunk = (j * 2 + (q >> 1)) ^ cswz(row);
                 u32x2_t w;
                 w[0] = cvt_store2<DT>(acc[i][j][0], acc[i][j][1]);
                 w[1] = cvt_store2<DT>(acc[i][j][2], acc[i][j][3]);
@@ -272,13 +362,31 @@ gemm_mfma16_kernel(const GemmArgs p) {
             }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        const int rr = lane / CPR, rc = lane % CPR;
-        const uint32_t cbase = (uint32_t)((wm * TM + rr) * p.ldc + col0 + wn * TN + rc * 8) * 2u;
 #pragma unroll
-        for (int r = 0; r < TM / RPI; ++r) {
-            const int row = r * RPI + rr;
-            const u32x4_t v = *(const u32x4_t*)(stg + row * (TN * 2) + ((rc ^ (row & (CPR - 1))) << 4));
-            __builtin_amdgcn_raw_buffer_store_b128(v, rsrcC, cbase + (uint32_t)(r * RPI * p.ldc) * 2u, 0, 0);
+        for (int r = 0; r < TM * CPR / 64; ++r) {
+            // chunk r*64 + lane of the wave tile, rows first
+            const int idx = r * 64 + lane;
+            const int row = POW2 ? r * (64 / CPR) + lane / CPR : idx / CPR;
+            const int rc = POW2 ? lane % CPR : idx % CPR;
+            const u32x4_t v = *(const u32x4_t*)(stg + row * (TN * 2) + ((rc ^ cswz(row)) << 4));
+            const int m_loc = wm * TM + row;
+            const int n = col0 + wn * TN + rc * 8;
+            const uint32_t off = (uint32_t)(m_loc * p.ldc + n) * 2u;
+            if constexpr (!EDGE) {
+                __builtin_amdgcn_raw_buffer_store_b128(v, rsrcC, off, 0, 0);
+            } else {
+                if (m_loc < rowsA) {
+                    if (n + 7 < N) {
+                        __builtin_amdgcn_raw_buffer_store_b128(v, rsrcC, off, 0, 0);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (n + e < N)
+                                __builtin_amdgcn_raw_buffer_store_b16(
+                                    (uint16_t)(v[e >> 1] >> ((e & 1) * 16)), rsrcC, off + 2 * e, 0, 0);
+                    }
+                }
+            }
         }
     }
     if constexpr (TRACE) {

@@ -78,9 +78,10 @@ class GemmTuner:
             'WN': [2, 4],
             'NS': [4],
             'SWZ': [1],
-            'GROUP': [4, 8, 16],
+            'GROUP': [4, 8],
             'DTL': [1],
             'EPI': [1],
+            'DRAIN': [0, 1, 3],
         }
 
         # Load template
@@ -156,6 +157,8 @@ class GemmTuner:
         c = dict(params, OCC=1)
         if c['KIND'] != 'tile' and (c.get('SWZ', 1) != 1 or c.get('DTL', 1) != 1 or c.get('EPI', 1) != 1):
             return False            # only the two-stage kernel has several load paths and epilogues
+        if c['KIND'] != 'mfma16' and c.get('DRAIN', 0) != 0:
+            return False            # the early drain barrier exists in the 16x16x32 two-stage kernel only
         if c['KIND'] in ('tile', 'mfma16') and c.get('NS', 4) != self.param_space['NS'][0]:
             return False            # NS is meaningless for the two-stage kernels: keep one copy
         try:

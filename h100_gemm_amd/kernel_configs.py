@@ -35,9 +35,7 @@ def config_name(c: dict) -> str:
     if c["KIND"] == "mfma16":
         name = f"m{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_g{c['GROUP']}"
         if c.get("DRAIN", 0):
-            name += "_b2"
-        if (c.get("EWM", c["WM"]), c.get("EWN", c["WN"])) != (c["WM"], c["WN"]):
-            name += f"_x{c['EWM']}x{c['EWN']}"
+            name += f"_b{c['DRAIN']}"
         return name
     if c["KIND"] == "ring16":
         return f"q{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_n{c['NS']}_g{c['GROUP']}"
@@ -68,7 +66,7 @@ def lds_bytes(c: dict) -> int:
 
 def is_valid_config(c: dict) -> bool:
     """Static rules of the kernels (mirrored as static_asserts in csrc/)."""
-    if c["KIND"] in ("ring", "mfma16", "ring16") and not c.get("_twin_checked"):
+    if c["KIND"] in ("ring", "ring16") and not c.get("_twin_checked"):
         # ragged shapes run the predicated two-stage kernel of the same tile and wave grid
         twin = dict(KIND="tile", BM=c["BM"], BN=c["BN"], WM=c.get("EWM", c["WM"]), WN=c.get("EWN", c["WN"]), SWZ=1,
                     GROUP=c["GROUP"], OCC=1, DTL=0, EPI=1)
@@ -113,8 +111,12 @@ def is_valid_config(c: dict) -> bool:
         if c["KIND"] == "ring16" and (c["NS"] != 4 or (c["NS"] - 1) * l > 63):
             return False
         tn = c["BN"] // c["WN"]
-        if tn & (tn - 1) or tn < 32:          # the C staging swizzle needs a power-of-two row
+        if tn < 32 or (c["KIND"] == "ring16" and tn & (tn - 1)):   # ring16: C staging needs a power-of-two row
             return False
+        if c["KIND"] == "mfma16" and c.get("DRAIN", 0):
+            sa = mi16 + ni16 + 4 * c["DRAIN"]
+            if sa + 1 >= mi16 * ni16 or (2 * mi16 * ni16 - 5 - sa) // l < 1:
+                return False
         if mi16 + ni16 + l > mi16 * ni16:
             return False
         return mi16 * ni16 * 4 + 2 * (mi16 + ni16) * 4 + 24 <= 512 // waves_per_simd
@@ -150,12 +152,10 @@ def _r(BM, BN, WM, WN, NS=4, GROUP=8):
     return dict(KIND="ring", BM=BM, BN=BN, WM=WM, WN=WN, NS=NS, GROUP=GROUP)
 
 
-def _m(BM, BN, WM, WN, GROUP=4, EFF=None, EW=None, DRAIN=0):
+def _m(BM, BN, WM, WN, GROUP=4, EFF=None, DRAIN=0):
     c = dict(KIND="mfma16", BM=BM, BN=BN, WM=WM, WN=WN, GROUP=GROUP)
     if DRAIN:
         c["DRAIN"] = DRAIN
-    if EW is not None:
-        c["EWM"], c["EWN"] = EW
     if EFF is not None:
         c["EFF"] = EFF
     return c
@@ -177,19 +177,22 @@ CONFIGS = [
     _c(256, 256, 2, 2, SWZ=1, GROUP=8),
     _c(256, 256, 2, 2, SWZ=1, GROUP=8, DTL=1),
     _c(256, 256, 2, 2, SWZ=1, GROUP=8, DTL=1, EPI=1),
-    _c(256, 256, 2, 2, SWZ=1, GROUP=4, DTL=1, EPI=1, EFF=0.9, EW=(2, 4)),
+    _c(256, 256, 2, 2, SWZ=1, GROUP=4, DTL=1, EPI=1, EW=(2, 4)),
     _c(256, 256, 2, 4, SWZ=1, GROUP=8, DTL=1, EPI=1),
     _c(256, 192, 2, 2, SWZ=1, GROUP=4, DTL=1, EPI=1),
-    _c(256, 192, 2, 2, SWZ=1, GROUP=4, DTL=1, EPI=1, EFF=0.89, EW=(4, 2)),
+    _c(256, 192, 2, 2, SWZ=1, GROUP=4, DTL=1, EPI=1, EW=(4, 2)),
     _c(256, 128, 2, 2, SWZ=1, GROUP=8, DTL=1, EPI=1, EW=(4, 2)),
     _c(128, 256, 2, 2, SWZ=1, GROUP=8, DTL=1, EPI=1, EW=(2, 4)),
-    _c(256, 128, 2, 2, SWZ=1, GROUP=8, DTL=1, EPI=1, EFF=0.81),
-    _c(128, 256, 2, 2, SWZ=1, GROUP=8, DTL=1, EPI=1, EFF=0.74),
-    _c(128, 128, 2, 2, SWZ=1, GROUP=8, OCC=2, DTL=1, EPI=1, EFF=0.83),
+    _c(256, 128, 2, 2, SWZ=1, GROUP=8, DTL=1, EPI=1),
+    _c(128, 256, 2, 2, SWZ=1, GROUP=8, DTL=1, EPI=1),
+    _c(128, 128, 2, 2, SWZ=1, GROUP=8, OCC=2, DTL=1, EPI=1, EFF=0.745),
     _r(256, 256, 2, 2),
     _r(256, 256, 2, 4),
-    _m(256, 256, 2, 2, EW=(2, 4)),
-    _m(256, 256, 2, 2, DRAIN=3, EFF=1.0, EW=(2, 4)),
+    _m(256, 256, 2, 2),
+    _m(256, 256, 2, 2, DRAIN=3, EFF=1.0),
+    _m(256, 192, 2, 2, DRAIN=3, EFF=0.89),
+    _m(128, 256, 2, 2, DRAIN=1, EFF=0.875),
+    _m(256, 128, 2, 2, DRAIN=1, EFF=0.845),
     _m(256, 256, 4, 2),
     _m(256, 256, 4, 2, DRAIN=3),
     _m(256, 256, 2, 4),
