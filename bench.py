@@ -48,10 +48,10 @@ WORKLOADS = {
 # FETCH_SIZE counts KiB and reads half of what a plain 256 MiB device copy moves (131087 for
 # 262144 KiB read), so it is scaled by 2.0; WRITE_SIZE reads the copy's writes exactly (1.0).
 MEASURED_TRAFFIC_BYTES = {
-    "square8192": (795438 * 2.0 + 131072) * 1024,     # 1.76 GB against 0.40 GB algorithmic
+    "square8192": (788687 * 2.0 + 131072) * 1024,     # 1.75 GB against 0.40 GB algorithmic
     "skinny16": (66589.6 * 2.0 + 256) * 1024,         # 0.137 GB: B is read exactly once
-    "unaligned": (129991 * 2.0 + 49716) * 1024,       # 0.317 GB against 0.113 GB algorithmic
-    "mlp_down": (2.758e6 * 2.0 + 141312) * 1024,      # 5.8 GB against 1.07 GB algorithmic
+    "unaligned": (130105 * 2.0 + 49737) * 1024,       # 0.317 GB against 0.113 GB algorithmic
+    "mlp_down": (2.7535e6 * 2.0 + 131072) * 1024,      # 5.8 GB against 1.07 GB algorithmic
     "skinny64": ((72064 + 3086) * 2.0 + 6144 + 1024) * 1024,     # main + reduce kernels
     "skinny128": ((80712 + 6158) * 2.0 + 12288 + 2048) * 1024,   # main + reduce kernels
 }
