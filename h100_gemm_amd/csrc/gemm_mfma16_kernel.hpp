@@ -1,21 +1,25 @@
-// gemm_mfma16_kernel.hpp -- aligned-shape gfx950 GEMM kernel built on
-// v_mfma_f32_16x16x32_{bf16,f16} with two waves per SIMD (8 waves per workgroup).
+// gemm_mfma16_kernel.hpp -- gfx950 GEMM kernels built on v_mfma_f32_16x16x32_{bf16,f16}:
+// the default tiled kernel of the library (aligned and predicated variants) and a ring variant.
 //
-//   C[M,N] = A[M,K] . B[N,K]^T     M % BM == 0, N % BN == 0, K % 128 == 0, 16-byte aligned
+//   C[M,N] = A[M,K] . B[N,K]^T
+//   aligned variant:    M % BM == 0, N % BN == 0, K % 128 == 0, 16-byte aligned pointers
+//   predicated variant: any M, N, K >= 1, any (2-byte) alignment
 //
-// Why a second MFMA shape: on random bf16 data the chip is power limited, and an MFMA-only
-// loop of 16x16x32 instructions sustains ~2.05 PFLOP/s where 32x32x16 sustains ~1.79 (the
-// 16x16 instruction moves half as many accumulator registers per flop).  The 4-pass
-// instruction needs two waves per SIMD to keep the pipe full, hence 512 threads and a
-// 128 x 64 (or 64 x 128) wave tile with 128 accumulator registers per lane.
+// Why this MFMA shape: on random bf16 data the chip is power limited, and an MFMA-only loop
+// of 16x16x32 instructions sustains ~1.9-2.05 PFLOP/s where 32x32x16 sustains ~1.75 (the
+// 16x16 instruction moves half as many accumulator registers per flop).  One wave per SIMD
+// issues it back to back (16.4 cycles per MFMA measured), so the kernel runs four waves with
+// a 128 x 128 wave tile (64 accumulator tiles, 256 AGPRs per lane) -- the least LDS traffic
+// per flop -- or eight waves with 64 x 128.
 //
 // Everything else follows gemm_kernel.hpp: two LDS stages of one 64-deep K slab each,
 // 128-byte rows with the 16-byte chunks stored at chunk ^ ((row >> 1) & 7), direct-to-LDS
-// buffer loads (inline asm, explicit waits), one barrier per K step, XCD-aware tile order,
-// C tile transposed through LDS and written 16 bytes per lane.  A K step is two 32-deep
-// slices: slice 0 multiplies while the fragments of slice 1 are fetched; after the barrier
-// slice 1 multiplies while slice 0 of the next slab is fetched and the loads of the slab
-// after that are issued.
+// buffer loads (inline asm, explicit waits), XCD-aware tile order, C tile transposed through
+// LDS and written 16 bytes per lane.  A K step is two 32-deep slices: slice 0 multiplies
+// while the fragments of slice 1 are fetched; after the mid-step barrier slice 1 multiplies
+// while slice 0 of the next slab is fetched.  The loads of the slab after next either go out
+// during slice 1 (DRAIN = 0) or, after an early second barrier that frees the current
+// stage, are spread over nearly the whole step (DRAIN > 0, see Mfma16Config).
 //
 // Fragment layout of the 16x16x32 MFMA: lane l holds row (l & 15), k chunk (l >> 4) of the
 // 32-deep slice (8 elements, 16 bytes); result register e of lane l is
