@@ -97,7 +97,8 @@ def all_configs(kinds=("tile", "ring", "mfma16", "ring16")):
 @pytest.mark.parametrize("config", all_configs())
 def test_every_config_bit_exact_on_integer_fill(mi, orc, config):
     # aligned (512^3: the aligned kernel), and ragged M, N, odd K (the predicated kernel)
-    for M, N, K in [(512, 512, 512), (768, 1536, 1152), (257, 515, 77), (300, 200, 136)]:
+    for M, N, K in [(512, 512, 512), (768, 1536, 1152), (257, 515, 77), (300, 200, 136), (65, 70, 33),
+                    (256, 384, 191), (1, 1, 1)]:
         check(mi, orc, M, N, K, "int", config=config, exact=True)
 
 
