@@ -86,11 +86,15 @@ def cpu_baseline(orc, A, B, budget_tiles: int) -> dict:
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    # The first ~100 launches after an idle period run 5-40 % slower while the power
+    # The first ~100 ms of launches after an idle period run 5-40 % slower while the power
     # management settles (per-launch durations in the kernel trace fall from ~1.1 ms to
-    # ~0.8 ms at 8192^3); the default warmup covers that transient.
+    # ~0.7 ms at 8192^3).  The default warmup covers that transient; --settle-ms keeps it
+    # covered when a caller passes a small --warmup: the same launches, untimed, for at least
+    # that long before the W warmup steps (reported as "settle_ms" in the JSON line).
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=150)
+    ap.add_argument("--settle-ms", type=float, default=150.0,
+                    help="untimed launches for at least this long before the warmup steps (0 = none)")
     ap.add_argument("--workload", default="square8192", choices=sorted(WORKLOADS))
     ap.add_argument("--config", default=None, help="kernel configuration name or index (default: library's choice)")
     ap.add_argument("--cpu-tiles", type=int, default=2048, help="64x64 tiles in the CPU baseline sample (0 = skip)")
@@ -140,6 +144,12 @@ def main() -> int:
         mi.synchronize()
         src.free()
         dst.free()
+    if a.settle_ms > 0:
+        t_end = time.perf_counter() + a.settle_ms * 1e-3
+        while time.perf_counter() < t_end:
+            for i in range(8):
+                mi.gpu_gemm(params[i % len(params)], config=cfg)
+            mi.synchronize()
     for i in range(a.warmup):
         mi.gpu_gemm(params[i % len(params)], config=cfg)
     mi.synchronize()
@@ -180,7 +190,7 @@ def main() -> int:
     out = {
         "metric": "bf16 GEMM TFLOP/s at M=N=K=8192 on 1 MI355X; % of bf16 MFMA peak",
         "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "settle_ms": a.settle_ms, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic" + (", 3 rotating copies of B" if hbm_bound else ""),
         "config": {"workload": f"{a.workload}: M={M} N={N} K={K}, A,B {fill} seeded bf16, fp32 accumulate, bf16 out",
                    "kernel_config": mi.config_name(cfg), "device": props["name"] or props["arch"],
