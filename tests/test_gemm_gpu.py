@@ -179,6 +179,52 @@ def test_misaligned_base_pointers(mi, orc):
     assert raw[0] == 0xEEEE and (raw[1 + M * N:] == 0xEEEE).all()      # nothing written outside C
 
 
+def _run_offset(mi, orc, config, M, N, K, offA, offB, offC, dtype=0):
+    """GEMM on sub-buffers that start offA/offB/offC bytes into their allocations; returns
+    (C, ref, guard words before and after C)."""
+    A, B = make_inputs(orc, M, N, K, "int", dtype)
+    ref = orc.reference_cpu_gemm(A, B, dtype=dtype)
+    dA = mi.DeviceBuffer(A.nbytes + 64)
+    dB = mi.DeviceBuffer(B.nbytes + 64)
+    dC = mi.DeviceBuffer(M * N * 2 + 128)
+    L = mi._lib.load()
+    mi._lib.check(L.mi_memcpy_h2d(dA.ptr + offA, A.ctypes.data, A.nbytes))
+    mi._lib.check(L.mi_memcpy_h2d(dB.ptr + offB, B.ctypes.data, B.nbytes))
+    dC.fill_bytes(0xEE)
+    mi._lib.check(L.mi_gemm_ex(config, dtype, M, N, K, dA.ptr + offA, dB.ptr + offB, dC.ptr + offC, None, None))
+    mi.synchronize()
+    raw = dC.to_numpy((M * N + 64,), np.uint16)
+    lo = offC // 2
+    C = raw[lo:lo + M * N].reshape(M, N)
+    guard = np.concatenate([raw[:lo], raw[lo + M * N:]])
+    for b in (dA, dB, dC):
+        b.free()
+    return C, ref, guard
+
+
+def test_random_shapes_and_alignments_every_tiled_kind(mi, orc):
+    # seeded sweep: ragged M, N, K (K tails of every length class, K < 64, K just above a
+    # multiple of 128), base pointers at arbitrary even byte offsets, through the automatic
+    # choice and through one configuration of every tiled kernel kind
+    from h100_gemm_amd import kernel_configs as kc
+    rng = np.random.default_rng(20240607)
+    picks = {}
+    for i, c in enumerate(kc.CONFIGS):
+        if c["KIND"] in ("tile", "ring", "mfma16", "ring16"):
+            picks.setdefault((c["KIND"], c.get("DRAIN", 0) > 0, c["BN"] == 192), i)
+    configs = [-1] + sorted(picks.values())
+    for it in range(36):
+        M = int(rng.integers(1, 700))
+        N = int(rng.integers(1, 700))
+        K = int(rng.choice([rng.integers(1, 64), rng.integers(64, 400), 128 * rng.integers(1, 5) + rng.integers(0, 9)]))
+        offA, offB, offC = (int(2 * rng.integers(0, 16)) for _ in range(3))
+        config = configs[it % len(configs)]
+        print(f"case {it}: M={M} N={N} K={K} offsets {offA},{offB},{offC} config={config}", flush=True)
+        C, ref, guard = _run_offset(mi, orc, config, M, N, K, offA, offB, offC)
+        assert (C == ref).all(), f"{int((C != ref).sum())} elements differ"
+        assert (guard == 0xEEEE).all(), "bytes outside C were written"
+
+
 def test_output_buffer_is_not_overrun(mi, orc):
     M, N, K = 257, 515, 77
     A, B = make_inputs(orc, M, N, K, "int")
