@@ -38,7 +38,7 @@ namespace mi {
 
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
-template <int BM_, int BN_, int WM_, int WN_, int GROUP_, int DT_, int DRAIN_ = 0, bool EDGE_ = false>
+template <int BM_, int BN_, int WM_, int WN_, int GROUP_, int DT_, int DRAIN_ = 0, bool EDGE_ = false, int OCC_ = 1>
 struct Mfma16Config {
     static constexpr int BM = BM_, BN = BN_, BK = 64;
     static constexpr int WM = WM_, WN = WN_, GROUP = GROUP_, DT = DT_;
@@ -51,9 +51,11 @@ struct Mfma16Config {
     static constexpr int LA = BM / RPP, LB = BN / RPP;   // load instructions per wave per slab
     static constexpr int A_STAGE = BM * 128, B_STAGE = BN * 128;
     static constexpr int LDS_BYTES = 2 * (A_STAGE + B_STAGE);
-    static constexpr int WAVES_PER_EU = NT / 256;
+    static constexpr int OCC = OCC_;                     // workgroups per CU the register / LDS budget is sized for
+    static constexpr int WAVES_PER_EU = NT / 256 * OCC;
     static constexpr int NMMA = MI * NI, NFR = MI + NI;
     static_assert(NT == 256 || NT == 512, "one or two waves per SIMD");
+    static_assert(OCC >= 1 && LDS_BYTES * OCC <= 160 * 1024, "LDS budget of one CU");
     static_assert(TM % 16 == 0 && TN % 16 == 0, "wave tile must be a multiple of 16x16");
     static_assert(BM % RPP == 0 && BN % RPP == 0 && RPP % 16 == 0, "tile rows divide over the threads");
     static constexpr int DSP = (NMMA - NFR) / (LA + LB);   // MFMA slots between two load instructions

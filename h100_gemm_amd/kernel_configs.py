@@ -8,7 +8,7 @@ template takes (matmul_h100.cu.jinja:9-14) -- re-cast for CDNA4:
     WM, WN   wave grid: WM*WN waves of 64 lanes, each owning a (BM/WM) x (BN/WN) sub-tile
     SWZ      LDS chunk swizzle (0: row & 7, 1: (row >> 1) & 7)
     GROUP    tile-order group height (L2 locality of the workgroups sharing an XCD)
-    OCC      workgroups per CU the register budget is sized for
+    OCC      workgroups per CU the register budget is sized for (tile and mfma16 kinds)
     DTL      1: direct-to-LDS global loads in the aligned kernel, 0: register staged
     KIND     "tile" (two-stage kernel above), "ring" (NS-deep LDS ring, K step 32, aligned
              shapes; ragged shapes take the predicated tile kernel of the same tile),
@@ -36,6 +36,8 @@ def config_name(c: dict) -> str:
         name = f"m{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_g{c['GROUP']}"
         if c.get("DRAIN", 0):
             name += f"_b{c['DRAIN']}"
+        if c.get("OCC", 1) != 1:
+            name += f"_o{c['OCC']}"
         return name
     if c["KIND"] == "ring16":
         return f"q{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_n{c['NS']}_g{c['GROUP']}"
@@ -152,8 +154,10 @@ def _r(BM, BN, WM, WN, NS=4, GROUP=8):
     return dict(KIND="ring", BM=BM, BN=BN, WM=WM, WN=WN, NS=NS, GROUP=GROUP)
 
 
-def _m(BM, BN, WM, WN, GROUP=4, EFF=None, DRAIN=0):
+def _m(BM, BN, WM, WN, GROUP=4, EFF=None, DRAIN=0, OCC=1):
     c = dict(KIND="mfma16", BM=BM, BN=BN, WM=WM, WN=WN, GROUP=GROUP)
+    if OCC != 1:
+        c["OCC"] = OCC
     if DRAIN:
         c["DRAIN"] = DRAIN
     if EFF is not None:
@@ -185,7 +189,7 @@ CONFIGS = [
     _c(128, 256, 2, 2, SWZ=1, GROUP=8, DTL=1, EPI=1, EW=(2, 4)),
     _c(256, 128, 2, 2, SWZ=1, GROUP=8, DTL=1, EPI=1),
     _c(128, 256, 2, 2, SWZ=1, GROUP=8, DTL=1, EPI=1),
-    _c(128, 128, 2, 2, SWZ=1, GROUP=8, OCC=2, DTL=1, EPI=1, EFF=0.745),
+    _c(128, 128, 2, 2, SWZ=1, GROUP=8, OCC=2, DTL=1, EPI=1),
     _r(256, 256, 2, 2),
     _r(256, 256, 2, 4),
     _m(256, 256, 2, 2),
@@ -193,6 +197,7 @@ CONFIGS = [
     _m(256, 192, 2, 2, DRAIN=3, EFF=0.89),
     _m(128, 256, 2, 2, DRAIN=1, EFF=0.875),
     _m(256, 128, 2, 2, DRAIN=1, EFF=0.845),
+    _m(128, 128, 2, 2, DRAIN=1, OCC=2, EFF=0.78),
     _m(256, 256, 4, 2),
     _m(256, 256, 4, 2, DRAIN=3),
     _m(256, 256, 2, 4),

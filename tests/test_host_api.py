@@ -121,6 +121,7 @@ def test_config_table(mi):
     assert picked(8192, 28672, 8192) == (256, 256)
     assert picked(4095, 6143, 3073) == (256, 192)
     assert picked(512, 512, 512) == (128, 128)
+    assert kc.CONFIGS[mi.select_config(512, 512, 512)]['KIND'] == 'mfma16'
     assert all("EFF" in kc.CONFIGS[mi.select_config(M, N, 4096)] for M in (129, 1000, 5000) for N in (100, 3000))
     assert not kc.is_valid_config(dict(KIND="tile", BM=256, BN=256, WM=2, WN=2, SWZ=1, GROUP=8, OCC=2, DTL=0, EPI=0))
     assert not kc.is_valid_config(dict(KIND="tile", BM=96, BN=256, WM=2, WN=2, SWZ=1, GROUP=8, OCC=1, DTL=0, EPI=0))
