@@ -82,6 +82,7 @@ class GemmTuner:
             'DTL': [1],
             'EPI': [1],
             'DRAIN': [0, 1, 3],
+            'OCC': [1, 2],
         }
 
         # Load template
@@ -100,7 +101,7 @@ class GemmTuner:
 
     @staticmethod
     def config_name(params: Dict[str, int]) -> str:
-        return kc.config_name(dict(params, OCC=1))
+        return kc.config_name(dict({'OCC': 1}, **params))
 
     def generate_code(self, params: Dict[str, int]) -> str:
         """Generate code with given parameters"""
@@ -154,9 +155,11 @@ class GemmTuner:
 
     def is_valid_configuration(self, params: Dict[str, int]) -> bool:
         """Check if a parameter configuration is valid"""
-        c = dict(params, OCC=1)
+        c = dict({'OCC': 1}, **params)
         if c['KIND'] != 'tile' and (c.get('SWZ', 1) != 1 or c.get('DTL', 1) != 1 or c.get('EPI', 1) != 1):
             return False            # only the two-stage kernel has several load paths and epilogues
+        if c['KIND'] in ('ring', 'ring16') and c.get('OCC', 1) != 1:
+            return False            # the ring kernels fill LDS with one workgroup
         if c['KIND'] != 'mfma16' and c.get('DRAIN', 0) != 0:
             return False            # the early drain barrier exists in the 16x16x32 two-stage kernel only
         if c['KIND'] in ('tile', 'mfma16') and c.get('NS', 4) != self.param_space['NS'][0]:
