@@ -350,7 +350,10 @@ void gpu_gemm(GemmParams<AType, BType, CType, AccumType> gemm_params, int config
 }
 
 // runKernel / run_kernel (matmul_h100_optimal.cu:32-59, 75-84).  kernel_num 1 is this
-// library's kernel; 0 is a vendor BLAS in the reference and is not linked here.
+// library's kernel.  0 is a vendor BLAS in the reference (runCublasGemmBF16,
+// matmul_h100_optimal.cu:63-73): the library links none, so a program that wants that arm
+// defines MI_HOST_VENDOR_GEMM to its own `void f(int M, int N, int K, void* A, void* B,
+// void* C)` before including this header (vendor_bench.cpp does, with hipBLASLt).
 inline void runKernel(int M, int N, int K, bf16* A, bf16* B, bf16* C, int* DB) {
     MI_CHECK(mi_gemm_bf16(M, N, K, (const uint16_t*)A, (const uint16_t*)B, (uint16_t*)C, DB, nullptr));
 }
@@ -358,6 +361,11 @@ inline void runKernel(int M, int N, int K, bf16* A, bf16* B, bf16* C, int* DB) {
 inline void run_kernel(int kernel_num, int M, int N, int K, bf16* A, bf16* B, bf16* C,
                        int* DB = nullptr) {
     switch (kernel_num) {
+#ifdef MI_HOST_VENDOR_GEMM
+        case 0:
+            MI_HOST_VENDOR_GEMM(M, N, K, (void*)A, (void*)B, (void*)C);
+            break;
+#endif
         case 1:
             runKernel(M, N, K, A, B, C, DB);
             break;

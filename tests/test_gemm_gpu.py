@@ -334,3 +334,17 @@ def test_harness_programs(mi):
     assert r.returncode == 0, r.stdout + r.stderr
     assert "KERNEL 1" in r.stdout
     assert re.search(r"Average elapsed time: \(\s*[\d.]+\) s, performance: \(\s*[\d.]+\) TFLOPS\. size: \(1024\)\.", r.stdout)
+
+
+def test_vendor_side_by_side_program(mi):
+    """kernel 0 (vendor BLAS, linked into this program only) and kernel 1 on the same buffers:
+    the loop of matmul_h100_optimal.cu:157-217 with the comparison of :177-180 switched on."""
+    exe = ROOT / "h100_gemm_amd" / "harness" / "vendor_bench"
+    if not exe.exists():
+        pytest.fail("vendor_bench is not built (make -C h100_gemm_amd/harness)")
+    for shape in (("512", "512", "512"), ("333", "257", "130"), ("16", "1024", "512")):
+        r = subprocess.run([str(exe), *shape, "3", "0"], capture_output=True, text=True, timeout=120)
+        assert r.returncode == 0, r.stdout + r.stderr
+        assert r.stdout.index("KERNEL 0") < r.stdout.index("KERNEL 1")
+        assert "Matches the vendor BLAS within tolerance." in r.stdout
+        assert len(re.findall(r"Average elapsed time: \(\s*[\d.]+\) s, performance: \(\s*[\d.]+\) TFLOPS\.", r.stdout)) == 2

@@ -30,6 +30,16 @@ def test_library_exports_every_declared_symbol(mi):
     assert set(names) == set(_lib.SYMBOLS), set(names) ^ set(_lib.SYMBOLS)
 
 
+def test_library_links_no_vendor_blas(mi):
+    """The vendor GEMM is a side-by-side program's business (harness/vendor_bench.cpp), never a
+    dispatch path of the library: its only run-time dependencies are HIP and the C/C++ runtime."""
+    from h100_gemm_amd import _lib
+    out = subprocess.run(["readelf", "-d", str(_lib.LIB_PATH)], capture_output=True, text=True, check=True).stdout
+    needed = re.findall(r"\(NEEDED\)\s+Shared library: \[([^\]]+)\]", out)
+    assert any(n.startswith("libamdhip64") for n in needed)
+    assert not [n for n in needed if re.search(r"blas|tensile|miopen|torch", n, re.I)], needed
+
+
 def test_missing_library_fails_loudly(mi, monkeypatch, tmp_path):
     from h100_gemm_amd import _lib
     monkeypatch.setattr(_lib, "_lib", None)
