@@ -20,9 +20,10 @@ from dataclasses import dataclass
 from typing import Any, Optional
 
 from . import _lib
-from ._lib import (MI_CONFIG_AUTO, MI_DTYPE_BF16, MI_DTYPE_FP16, DeviceProps, MiGemmError)
+from ._lib import (MI_C_COL_MAJOR, MI_C_ROW_MAJOR, MI_CONFIG_AUTO, MI_DTYPE_BF16, MI_DTYPE_FP16, DeviceProps,
+                   MiGemmError)
 
-__all__ = ["runKernel", "run_kernel", "gpu_gemm", "reference_gpu_gemm", "GemmParams", "DeviceBuffer", "GPUTimer",
+__all__ = ["runKernel", "run_kernel", "gpu_gemm", "gemm_epilogue", "MI_C_ROW_MAJOR", "MI_C_COL_MAJOR", "reference_gpu_gemm", "GemmParams", "DeviceBuffer", "GPUTimer",
            "device_props", "num_configs", "config_name", "find_config", "select_config",
            "config_grid", "synchronize", "MiGemmError", "MI_CONFIG_AUTO", "MI_DTYPE_BF16",
            "MI_DTYPE_FP16"]
@@ -51,8 +52,8 @@ def _stream(s: Any) -> Optional[int]:
 @dataclass
 class GemmParams:
     """The reference's GemmParams (common.h:206-221).  alpha/beta are carried for parity of
-    the signature; like the reference kernels (matmul_h100.cu.jinja:696) the GPU path
-    computes alpha = 1, beta = 0 and rejects anything else."""
+    the signature; like the reference kernels (matmul_h100.cu.jinja:696) ``gpu_gemm``
+    computes alpha = 1, beta = 0 and rejects anything else; ``gemm_epilogue`` honours both."""
     M: int
     N: int
     K: int
@@ -83,15 +84,32 @@ def gpu_gemm(params: GemmParams, config: int | str = MI_CONFIG_AUTO, dtype: int 
     """gpu_gemm<...>(GemmParams) of matmul_h100.cu.jinja:927-985; the template arguments
     become ``config`` (index or name of a compiled kernel configuration) and ``dtype``."""
     if params.alpha != 1.0 or params.beta != 0.0:
-        raise ValueError("the GPU path computes alpha = 1, beta = 0 only")
+        raise ValueError("gpu_gemm computes alpha = 1, beta = 0 only (as the reference's kernels do); "
+                         "gemm_epilogue applies alpha and beta")
     L = _lib.load()
+    config = _config_index(L, config)
+    _lib.check(L.mi_gemm_ex(config, dtype, params.M, params.N, params.K, _ptr(params.A),
+                            _ptr(params.B), _ptr(params.C), _ptr(DB), _stream(stream)))
+
+
+def _config_index(L, config) -> int:
     if isinstance(config, str):
         idx = L.mi_gemm_find_config(config.encode())
         if idx < 0:
             raise ValueError(f"unknown kernel config {config!r}")
-        config = idx
-    _lib.check(L.mi_gemm_ex(config, dtype, params.M, params.N, params.K, _ptr(params.A),
-                            _ptr(params.B), _ptr(params.C), _ptr(DB), _stream(stream)))
+        return idx
+    return config
+
+
+def gemm_epilogue(params: GemmParams, config: int | str = MI_CONFIG_AUTO, dtype: int = MI_DTYPE_BF16,
+                  c_layout: int = MI_C_ROW_MAJOR, stream=None) -> None:
+    """The GEMM with the golden's epilogue, C = (CType)(acc * alpha + beta) with beta a plain
+    scalar (reference.h:40), and C row-major or column-major (C[n*M + m], the layout the
+    reference's bf16 kernel writes, matmul_utils.cuh:529,545)."""
+    L = _lib.load()
+    _lib.check(L.mi_gemm_epilogue(_config_index(L, config), dtype, params.M, params.N, params.K,
+                                  _ptr(params.A), _ptr(params.B), _ptr(params.C), params.alpha,
+                                  params.beta, c_layout, _stream(stream)))
 
 
 def reference_gpu_gemm(params: GemmParams, dtype: int = MI_DTYPE_BF16, stream=None) -> None:

@@ -17,6 +17,8 @@ MI_ERR_UNSUPPORTED = -3
 MI_DTYPE_BF16 = 0
 MI_DTYPE_FP16 = 1
 MI_CONFIG_AUTO = -1
+MI_C_ROW_MAJOR = 0
+MI_C_COL_MAJOR = 1
 
 
 class MiGemmError(RuntimeError):
@@ -38,6 +40,8 @@ SYMBOLS = {
                                C.c_void_p, C.c_void_p]),
     "mi_gemm_ex": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
                              C.c_void_p, C.c_void_p, C.c_void_p]),
+    "mi_gemm_epilogue": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
+                                   C.c_void_p, C.c_float, C.c_float, C.c_int, C.c_void_p]),
     "mi_reference_gpu_gemm": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
                                         C.c_void_p, C.c_float, C.c_float, C.c_void_p]),
     "mi_gemm_num_configs": (C.c_int, []),

@@ -56,6 +56,8 @@ struct GemmArgs {
     int* DB;                 // optional trace buffer (may be null)
     float* ws;               // split-K workspace (decode kernels only)
     int splits, k_per_split; // split-K geometry (decode kernels only)
+    float alpha = 1.0f;      // C = (CType)(acc * alpha + beta), beta a plain scalar added to
+    float beta = 0.0f;       // every element (reference.h:40)
 };
 
 // Compile-time description of one kernel variant -- the knobs the tuner sweeps.
@@ -127,6 +129,18 @@ __device__ __forceinline__ uint32_t cvt_store2(float lo, float hi) {
 // __syncthreads(): that also drains vmcnt and would serialise the global prefetch.
 __device__ __forceinline__ void lds_barrier() {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// The epilogue of the reference's golden (reference.h:40): C = (CType)(acc * alpha + beta),
+// two separately rounded fp32 operations, beta a plain scalar added to every element.
+// alpha = 1, beta = 0 is what the reference's kernels compute (matmul_h100.cu.jinja:696) and
+// what SCALED = false leaves out entirely: the kernels hold two copies of their epilogue
+// behind one uniform branch, so the unscaled path and the K loop are unchanged by it.
+// (Scaling the accumulators in place before a single epilogue costs registers in the loop.)
+template <bool SCALED>
+__device__ __forceinline__ float scale_acc(float x, float alpha, float beta) {
+    if constexpr (SCALED) return __fadd_rn(__fmul_rn(x, alpha), beta);
+    else return x;
 }
 
 // blockIdx -> (tile_m, tile_n).  Hardware deals consecutive workgroup ids round-robin to
@@ -553,6 +567,9 @@ gemm_tile_kernel(const GemmArgs p) {
     const uint32_t bytesC = (uint32_t)(rowsA * p.ldc) * 2u;
     const __amdgpu_buffer_rsrc_t rsrcC =
         __builtin_amdgcn_make_buffer_rsrc((void*)Cb, 0, (int)bytesC, 0x00020000);
+    auto epilogue = [&](auto scaled_c) __attribute__((always_inline)) {
+    constexpr bool SCALED = decltype(scaled_c)::value;   // alpha / beta epilogue: see scale_acc
+    const float alpha = p.alpha, beta = p.beta;
     if constexpr (Cfg::EPI) {
         // Through LDS: each wave lays its TM x TN tile out row-major in its own slice of the
         // (now idle) stage buffers, 16-byte chunks XOR-swizzled by the row, then reads rows
@@ -581,8 +598,10 @@ gemm_tile_kernel(const GemmArgs p) {
                 for (int g = 0; g < 4; ++g) {
                     const int chunk = (j * 4 + g) ^ cswz(row);
                     u32x2_t w;
-                    w[0] = cvt_store2<DT>(acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1]);
-                    w[1] = cvt_store2<DT>(acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]);
+                    w[0] = cvt_store2<DT>(scale_acc<SCALED>(acc[i][j][g * 4 + 0], alpha, beta),
+                                          scale_acc<SCALED>(acc[i][j][g * 4 + 1], alpha, beta));
+                    w[1] = cvt_store2<DT>(scale_acc<SCALED>(acc[i][j][g * 4 + 2], alpha, beta),
+                                          scale_acc<SCALED>(acc[i][j][g * 4 + 3], alpha, beta));
                     *(u32x2_t*)(stg + row * (TN * 2) + chunk * 16 + hi * 8) = w;
                 }
             }
@@ -624,8 +643,10 @@ gemm_tile_kernel(const GemmArgs p) {
             for (int g = 0; g < 4; ++g) {
                 const int n = col0 + wn * Cfg::TN + j * 32 + g * 8 + hi * 4;
                 const uint32_t off = (uint32_t)(m_loc * p.ldc + n) * 2u;
-                const float v0 = acc[i][j][g * 4 + 0], v1 = acc[i][j][g * 4 + 1];
-                const float v2 = acc[i][j][g * 4 + 2], v3 = acc[i][j][g * 4 + 3];
+                const float v0 = scale_acc<SCALED>(acc[i][j][g * 4 + 0], alpha, beta);
+                const float v1 = scale_acc<SCALED>(acc[i][j][g * 4 + 1], alpha, beta);
+                const float v2 = scale_acc<SCALED>(acc[i][j][g * 4 + 2], alpha, beta);
+                const float v3 = scale_acc<SCALED>(acc[i][j][g * 4 + 3], alpha, beta);
                 if constexpr (!EDGE) {
                     u32x2_t w;
                     w[0] = cvt_store2<DT>(v0, v1);
@@ -650,6 +671,9 @@ gemm_tile_kernel(const GemmArgs p) {
         }
     }
     }
+    };
+    if (p.alpha != 1.0f || p.beta != 0.0f) epilogue(std::true_type{});
+    else epilogue(std::false_type{});
     if constexpr (TRACE) {
         if (p.DB != nullptr && tid == 0) {
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the stores have left the wave

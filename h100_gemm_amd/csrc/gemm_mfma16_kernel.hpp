@@ -342,7 +342,10 @@ gemm_mfma16_kernel(const GemmArgs p) {
     unsigned char* Cb = (unsigned char*)p.C + (size_t)row0 * p.ldc * 2;
     const uint32_t bytesC = (uint32_t)(rowsA * p.ldc) * 2u;
     const __amdgpu_buffer_rsrc_t rsrcC = __builtin_amdgcn_make_buffer_rsrc((void*)Cb, 0, (int)bytesC, 0x00020000);
-    {
+    auto epilogue = [&](auto scaled_c) __attribute__((always_inline)) {
+        // alpha / beta epilogue (see scale_acc): a second copy of this block behind a uniform branch
+        constexpr bool SCALED = decltype(scaled_c)::value;
+        const float alpha = p.alpha, beta = p.beta;
         // The predicated variant masks rows past M, stores 16 bytes at any 2-byte boundary
         // (odd N) and splits only the chunk that straddles N into 2-byte stores.
         // C is written once and not read again here: in the aligned variant non-temporal stores
@@ -368,8 +371,8 @@ gemm_mfma16_kernel(const GemmArgs p) {
             for (int j = 0; j < NI; ++j) {
                 const int chunk = (j * 2 + (q >> 1)) ^ cswz(row);
                 u32x2_t w;
-                w[0] = cvt_store2<DT>(acc[i][j][0], acc[i][j][1]);
-                w[1] = cvt_store2<DT>(acc[i][j][2], acc[i][j][3]);
+                w[0] = cvt_store2<DT>(scale_acc<SCALED>(acc[i][j][0], alpha, beta), scale_acc<SCALED>(acc[i][j][1], alpha, beta));
+                w[1] = cvt_store2<DT>(scale_acc<SCALED>(acc[i][j][2], alpha, beta), scale_acc<SCALED>(acc[i][j][3], alpha, beta));
                 *(u32x2_t*)(stg + row * (TN * 2) + chunk * 16 + (q & 1) * 8) = w;
             }
         }
@@ -400,7 +403,9 @@ gemm_mfma16_kernel(const GemmArgs p) {
                 }
             }
         }
-    }
+    };
+    if (p.alpha != 1.0f || p.beta != 0.0f) epilogue(std::true_type{});
+    else epilogue(std::false_type{});
     if constexpr (TRACE) {
         if (p.DB != nullptr && tid == 0) {
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -583,7 +588,9 @@ gemm_ring16_kernel(const GemmArgs p) {
     unsigned char* Cb = (unsigned char*)p.C + (size_t)row0 * p.ldc * 2;
     const uint32_t bytesC = (uint32_t)(BM * p.ldc) * 2u;
     const __amdgpu_buffer_rsrc_t rsrcC = __builtin_amdgcn_make_buffer_rsrc((void*)Cb, 0, (int)bytesC, 0x00020000);
-    {
+    auto epilogue = [&](auto scaled_c) __attribute__((always_inline)) {
+        constexpr bool SCALED = decltype(scaled_c)::value;   // alpha / beta epilogue: second copy behind a uniform branch
+        const float alpha = p.alpha, beta = p.beta;
         constexpr int CPR = TN / 8;
         constexpr int RPI = 64 / CPR;
         unsigned char* stg = lds + wave * (TM * TN * 2);
@@ -594,8 +601,8 @@ gemm_ring16_kernel(const GemmArgs p) {
             for (int j = 0; j < NI; ++j) {
                 const int chunk = (j * 2 + (q >> 1)) ^ (row & (CPR - 1));
                 u32x2_t w;
-                w[0] = cvt_store2<DT>(acc[i][j][0], acc[i][j][1]);
-                w[1] = cvt_store2<DT>(acc[i][j][2], acc[i][j][3]);
+                w[0] = cvt_store2<DT>(scale_acc<SCALED>(acc[i][j][0], alpha, beta), scale_acc<SCALED>(acc[i][j][1], alpha, beta));
+                w[1] = cvt_store2<DT>(scale_acc<SCALED>(acc[i][j][2], alpha, beta), scale_acc<SCALED>(acc[i][j][3], alpha, beta));
                 *(u32x2_t*)(stg + row * (TN * 2) + chunk * 16 + (q & 1) * 8) = w;
             }
         }
@@ -608,7 +615,9 @@ gemm_ring16_kernel(const GemmArgs p) {
             const u32x4_t v = *(const u32x4_t*)(stg + row * (TN * 2) + ((rc ^ (row & (CPR - 1))) << 4));
             __builtin_amdgcn_raw_buffer_store_b128(v, rsrcC, cbase + (uint32_t)(r * RPI * p.ldc) * 2u, 0, 0);
         }
-    }
+    };
+    if (p.alpha != 1.0f || p.beta != 0.0f) epilogue(std::true_type{});
+    else epilogue(std::false_type{});
     if constexpr (TRACE) {
         if (p.DB != nullptr && tid == 0) {
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");

@@ -45,6 +45,8 @@ struct SkinnyArgs {
     int lda, ldb, ldc;
     int k_per_split;      // unused by the kernels (host bookkeeping)
     int splits;           // <= K / 64
+    float alpha = 1.0f;   // C = (CType)(acc * alpha + beta), applied where the sum over K is
+    float beta = 0.0f;    // complete
 };
 
 template <int BM_, int BN_, int NS_, int DT_>
@@ -214,6 +216,7 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(const SkinnyArgs p) {
 
     // ---- epilogue: lane holds C[m][n..n+3], m = i*32 + (lane & 31), n = 8g + 4*(lane>>5) ----
     if (S == 1) {
+        const bool scaled = p.alpha != 1.0f || p.beta != 0.0f;
         unsigned char* Cb = (unsigned char*)p.C;
         const __amdgpu_buffer_rsrc_t rsrcC =
             __builtin_amdgcn_make_buffer_rsrc((void*)Cb, 0, (int)((uint32_t)(M * p.ldc) * 2u), 0x00020000);
@@ -227,8 +230,14 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(const SkinnyArgs p) {
                     const int n = col0 + wn * TN + j * 32 + g * 8 + hi * 4;
                     if (m < M && n < N) {           // N % 4 == 0 is a launch precondition
                         u32x2_t w;
-                        w[0] = cvt_store2<DT>(acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1]);
-                        w[1] = cvt_store2<DT>(acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]);
+                        float v[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            v[e] = acc[i][j][g * 4 + e];
+                            if (scaled) v[e] = scale_acc<true>(v[e], p.alpha, p.beta);
+                        }
+                        w[0] = cvt_store2<DT>(v[0], v[1]);
+                        w[1] = cvt_store2<DT>(v[2], v[3]);
                         __builtin_amdgcn_raw_buffer_store_b64(w, rsrcC, (uint32_t)(m * p.ldc + n) * 2u, 0, 0);
                     }
                 }
@@ -253,10 +262,11 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(const SkinnyArgs p) {
     }
 }
 
-// C[m][n] = round(sum over splits, in split order, of ws[s][m][n]); 4 elements per thread.
+// C[m][n] = round(alpha * (sum over splits, in split order, of ws[s][m][n]) + beta); 4 elements per thread.
 template <int DT>
 __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restrict__ ws, void* C, int M,
-                                                            int N, int ldc, int splits) {
+                                                            int N, int ldc, int splits, float alpha,
+                                                            float beta) {
     const size_t idx = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
     const size_t total = (size_t)M * N;
     if (idx >= total) return;
@@ -264,6 +274,12 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restr
     for (int s = 1; s < splits; ++s) {
         const float4 b = *(const float4*)(ws + (size_t)s * total + idx);
         a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+    }
+    if (alpha != 1.0f || beta != 0.0f) {
+        a.x = __fadd_rn(__fmul_rn(a.x, alpha), beta);
+        a.y = __fadd_rn(__fmul_rn(a.y, alpha), beta);
+        a.z = __fadd_rn(__fmul_rn(a.z, alpha), beta);
+        a.w = __fadd_rn(__fmul_rn(a.w, alpha), beta);
     }
     const size_t m = idx / N, n = idx % N;
     u32x2_t w;
@@ -280,7 +296,7 @@ hipError_t launch_skinny_kernel(const SkinnyArgs& a, hipStream_t stream) {
     if (e != hipSuccess || a.splits == 1) return e;
     const size_t quads = ((size_t)a.M * a.N + 3) / 4;
     hipLaunchKernelGGL((splitk_reduce_kernel<Cfg::DT>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0,
-                       stream, a.ws, a.C, a.M, a.N, a.ldc, a.splits);
+                       stream, a.ws, a.C, a.M, a.N, a.ldc, a.splits, a.alpha, a.beta);
     return hipGetLastError();
 }
 

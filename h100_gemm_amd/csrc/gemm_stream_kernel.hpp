@@ -166,6 +166,12 @@ __global__ void __launch_bounds__(256) gemm_stream_kernel(const SkinnyArgs p) {
             const float4 v = *(const float4*)((const float*)(lds + w * RING) + m * 32 + n);
             sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
         }
+        if (p.alpha != 1.0f || p.beta != 0.0f) {
+            sum.x = __fadd_rn(__fmul_rn(sum.x, p.alpha), p.beta);
+            sum.y = __fadd_rn(__fmul_rn(sum.y, p.alpha), p.beta);
+            sum.z = __fadd_rn(__fmul_rn(sum.z, p.alpha), p.beta);
+            sum.w = __fadd_rn(__fmul_rn(sum.w, p.alpha), p.beta);
+        }
         if (m < M && col0 + n < N) {                         // N % 4 == 0 is a launch precondition
             u32x2_t w2;
             w2[0] = cvt_store2<DT>(sum.x, sum.y);

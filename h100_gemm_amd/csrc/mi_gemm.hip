@@ -132,6 +132,74 @@ int check_args(int config, int dtype, int M, int N, int K, const void* A, const 
     return MI_OK;
 }
 
+// One GEMM launch (two for split-K): argument checks, kernel choice, aligned / predicated twin.
+int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const void* B, void* C,
+             int* DB, float alpha, float beta, void* stream) {
+    int rc = check_args(config, dtype, M, N, K, A, B, C);
+    if (rc != MI_OK) return rc;
+    const bool streamable = shape_is_streamable(M, N, K, A, B, C);
+    if (config == MI_CONFIG_AUTO) config = mi::select_kernel(M, N, K, streamable, compute_units());
+    const mi::KernelEntry& e = mi::kKernels[config];
+
+    mi::GemmArgs args;
+    args.A = A;
+    args.B = B;
+    args.C = C;
+    args.M = M;
+    args.N = N;
+    args.K = K;
+    args.lda = K;
+    args.ldb = K;
+    args.ldc = N;
+    args.tiles_m = (M + e.BM - 1) / e.BM;
+    args.tiles_n = (N + e.BN - 1) / e.BN;
+    args.c_vec_ok = (N % 4 == 0) && (((uintptr_t)C & 7u) == 0);
+    args.DB = DB;
+    args.ws = nullptr;
+    args.splits = 1;
+    args.k_per_split = K;
+    args.alpha = alpha;
+    args.beta = beta;
+
+    if (e.kind == mi::KIND_STREAM) {
+        if (!streamable || M > e.BM)
+            return fail(MI_ERR_UNSUPPORTED,
+                        "config %s needs M <= %d, N %% 4 == 0, K %% 64 == 0 and 16-byte aligned operands",
+                        e.name, e.BM);
+        hipError_t err = e.launch[dtype][0](args, (hipStream_t)stream);
+        if (err != hipSuccess)
+            return fail(MI_ERR_HIP, "launch of %s failed: %s", e.name, hipGetErrorString(err));
+        return MI_OK;
+    }
+    if (e.kind == mi::KIND_SKINNY) {
+        if (!streamable || M > e.BM)
+            return fail(MI_ERR_UNSUPPORTED,
+                        "config %s needs M <= %d, N %% 4 == 0, K %% 64 == 0 and 16-byte aligned operands",
+                        e.name, e.BM);
+        const int tiles_n = (N + e.BN - 1) / e.BN;
+        args.splits = choose_splits(tiles_n, K, compute_units(), e.lds_bytes);   // <= K / 64: no empty split
+        args.k_per_split = ((K / 64 + args.splits - 1) / args.splits) * 64;
+        if (args.splits > 1) {
+            hipError_t we = ensure_workspace((size_t)args.splits * M * N * sizeof(float), &args.ws);
+            if (we != hipSuccess)
+                return fail(MI_ERR_HIP, "split-K workspace allocation failed: %s", hipGetErrorString(we));
+        }
+        hipError_t err = e.launch[dtype][0](args, (hipStream_t)stream);
+        if (err != hipSuccess)
+            return fail(MI_ERR_HIP, "launch of %s failed: %s", e.name, hipGetErrorString(err));
+        return MI_OK;
+    }
+
+    const bool edge = !shape_is_aligned(e, M, N, K, A, B, C);
+    mi::LaunchFn fn = e.launch[dtype][edge ? 1 : 0];
+    if (!fn) return fail(MI_ERR_UNSUPPORTED, "config %s has no %s kernel for dtype %d", e.name,
+                         edge ? "predicated" : "aligned", dtype);
+    hipError_t err = fn(args, (hipStream_t)stream);
+    if (err != hipSuccess)
+        return fail(MI_ERR_HIP, "launch of %s failed: %s", e.name, hipGetErrorString(err));
+    return MI_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -197,67 +265,20 @@ size_t mi_gemm_trace_words(int M, int N, int K) {
 
 int mi_gemm_ex(int config, int dtype, int M, int N, int K, const void* A, const void* B,
                void* C, int* DB, void* stream) {
-    int rc = check_args(config, dtype, M, N, K, A, B, C);
-    if (rc != MI_OK) return rc;
-    const bool streamable = shape_is_streamable(M, N, K, A, B, C);
-    if (config == MI_CONFIG_AUTO) config = mi::select_kernel(M, N, K, streamable, compute_units());
-    const mi::KernelEntry& e = mi::kKernels[config];
+    return run_gemm(config, dtype, M, N, K, A, B, C, DB, 1.0f, 0.0f, stream);
+}
 
-    mi::GemmArgs args;
-    args.A = A;
-    args.B = B;
-    args.C = C;
-    args.M = M;
-    args.N = N;
-    args.K = K;
-    args.lda = K;
-    args.ldb = K;
-    args.ldc = N;
-    args.tiles_m = (M + e.BM - 1) / e.BM;
-    args.tiles_n = (N + e.BN - 1) / e.BN;
-    args.c_vec_ok = (N % 4 == 0) && (((uintptr_t)C & 7u) == 0);
-    args.DB = DB;
-    args.ws = nullptr;
-    args.splits = 1;
-    args.k_per_split = K;
-
-    if (e.kind == mi::KIND_STREAM) {
-        if (!streamable || M > e.BM)
-            return fail(MI_ERR_UNSUPPORTED,
-                        "config %s needs M <= %d, N %% 4 == 0, K %% 64 == 0 and 16-byte aligned operands",
-                        e.name, e.BM);
-        hipError_t err = e.launch[dtype][0](args, (hipStream_t)stream);
-        if (err != hipSuccess)
-            return fail(MI_ERR_HIP, "launch of %s failed: %s", e.name, hipGetErrorString(err));
-        return MI_OK;
-    }
-    if (e.kind == mi::KIND_SKINNY) {
-        if (!streamable || M > e.BM)
-            return fail(MI_ERR_UNSUPPORTED,
-                        "config %s needs M <= %d, N %% 4 == 0, K %% 64 == 0 and 16-byte aligned operands",
-                        e.name, e.BM);
-        const int tiles_n = (N + e.BN - 1) / e.BN;
-        args.splits = choose_splits(tiles_n, K, compute_units(), e.lds_bytes);   // <= K / 64: no empty split
-        args.k_per_split = ((K / 64 + args.splits - 1) / args.splits) * 64;
-        if (args.splits > 1) {
-            hipError_t we = ensure_workspace((size_t)args.splits * M * N * sizeof(float), &args.ws);
-            if (we != hipSuccess)
-                return fail(MI_ERR_HIP, "split-K workspace allocation failed: %s", hipGetErrorString(we));
-        }
-        hipError_t err = e.launch[dtype][0](args, (hipStream_t)stream);
-        if (err != hipSuccess)
-            return fail(MI_ERR_HIP, "launch of %s failed: %s", e.name, hipGetErrorString(err));
-        return MI_OK;
-    }
-
-    const bool edge = !shape_is_aligned(e, M, N, K, A, B, C);
-    mi::LaunchFn fn = e.launch[dtype][edge ? 1 : 0];
-    if (!fn) return fail(MI_ERR_UNSUPPORTED, "config %s has no %s kernel for dtype %d", e.name,
-                         edge ? "predicated" : "aligned", dtype);
-    hipError_t err = fn(args, (hipStream_t)stream);
-    if (err != hipSuccess)
-        return fail(MI_ERR_HIP, "launch of %s failed: %s", e.name, hipGetErrorString(err));
-    return MI_OK;
+int mi_gemm_epilogue(int config, int dtype, int M, int N, int K, const void* A, const void* B,
+                     void* C, float alpha, float beta, int c_layout, void* stream) {
+    if (c_layout != MI_C_ROW_MAJOR && c_layout != MI_C_COL_MAJOR)
+        return fail(MI_ERR_INVALID, "unknown C layout %d", c_layout);
+    if (!(alpha == alpha) || !(beta == beta)) return fail(MI_ERR_INVALID, "alpha or beta is NaN");
+    // Column-major C (M x N, element (m, n) at C[n*M + m]) is the row-major N x M matrix
+    // C^T = B . A^T: the same GEMM with the operands and their extents exchanged.  Every
+    // element is still the k-ordered sum the kernels form for the row-major case.
+    if (c_layout == MI_C_COL_MAJOR)
+        return run_gemm(config, dtype, N, M, K, B, A, C, nullptr, alpha, beta, stream);
+    return run_gemm(config, dtype, M, N, K, A, B, C, nullptr, alpha, beta, stream);
 }
 
 int mi_gemm_bf16(int M, int N, int K, const uint16_t* A, const uint16_t* B, uint16_t* C, int* DB,

@@ -38,6 +38,9 @@ extern "C" {
 
 #define MI_CONFIG_AUTO (-1)
 
+#define MI_C_ROW_MAJOR 0 /* element (m, n) of C at C[m*N + n] */
+#define MI_C_COL_MAJOR 1 /* element (m, n) of C at C[n*M + m] */
+
 /* ---- the GEMM ---------------------------------------------------------------------- */
 
 /* bf16 GEMM with the library's own choice of kernel for the shape.
@@ -55,6 +58,18 @@ int mi_gemm_bf16(int M, int N, int K, const uint16_t* A, const uint16_t* B, uint
  * MI_CONFIG_AUTO) and `dtype` (MI_DTYPE_*). */
 int mi_gemm_ex(int config, int dtype, int M, int N, int K, const void* A, const void* B,
                void* C, int* DB, void* stream);
+
+/* The same GEMM with the epilogue and the C layouts of the reference's other code paths:
+ *     C = (CType)(acc * alpha + beta)
+ * as two separately rounded fp32 operations with beta a plain scalar added to every
+ * element -- the epilogue of the reference's golden (reference.h:40, :69-76), which its
+ * hand-written kernels skip (matmul_h100.cu.jinja:696) -- and C either row-major
+ * (reference.h:40, matmul_h100.cu.jinja:696) or column-major, C[n*M + m], which is how the
+ * bf16 kernel behind runKernel stores it (matmul_utils.cuh:529,545).  alpha = 1, beta = 0,
+ * MI_C_ROW_MAJOR is exactly mi_gemm_ex without a trace buffer.  Column-major runs the
+ * kernels on the exchanged operands (C^T = B . A^T), so the kernel is chosen for N x M x K. */
+int mi_gemm_epilogue(int config, int dtype, int M, int N, int K, const void* A, const void* B,
+                     void* C, float alpha, float beta, int c_layout, void* stream);
 
 /* Plain, order-preserving GPU GEMM used as golden by the harness: one fp32 accumulator per
  * element fed in ascending k, C = (CType)(acc * alpha + beta), beta a scalar.

@@ -36,6 +36,13 @@ class Dev:
         self.mi.synchronize()
         return self.dC.to_numpy((self.M, self.N), np.uint16)
 
+    def run_epilogue(self, K, alpha, beta, c_layout=0, config=-1, dtype=0):
+        p = self.mi.GemmParams(self.M, self.N, K, self.dA, self.dB, self.dC, alpha, beta)
+        self.mi.gemm_epilogue(p, config=config, dtype=dtype, c_layout=c_layout)
+        self.mi.synchronize()
+        shape = (self.N, self.M) if c_layout == self.mi.MI_C_COL_MAJOR else (self.M, self.N)
+        return self.dC.to_numpy(shape, np.uint16)
+
 
 def make_inputs(orc, M, N, K, fill, dtype=0, seed=69):
     if fill == "uniform":
@@ -348,3 +355,79 @@ def test_vendor_side_by_side_program(mi):
         assert r.stdout.index("KERNEL 0") < r.stdout.index("KERNEL 1")
         assert "Matches the vendor BLAS within tolerance." in r.stdout
         assert len(re.findall(r"Average elapsed time: \(\s*[\d.]+\) s, performance: \(\s*[\d.]+\) TFLOPS\.", r.stdout)) == 2
+
+
+# ------------------------------- alpha / beta epilogue and column-major C (mi_gemm_epilogue) ----
+
+def check_epilogue(mi, orc, M, N, K, fill, alpha, beta, c_layout=0, config=-1, dtype=0, exact=False):
+    """C = storage(acc * alpha + beta), beta a plain scalar (reference.h:40); column-major C is
+    C[n*M + m] (matmul_utils.cuh:545), i.e. the transpose of the oracle's row-major result.
+    Tolerance: the benchmark bound with its absolute term scaled by |alpha|."""
+    print(f"case epilogue M={M} N={N} K={K} fill={fill} alpha={alpha} beta={beta} layout={c_layout} "
+          f"config={config} dtype={dtype}", flush=True)
+    A, B = make_inputs(orc, M, N, K, fill, dtype)
+    C = Dev(mi, A, B, M, N).run_epilogue(K, alpha, beta, c_layout, config, dtype)
+    ref = orc.reference_cpu_gemm(A, B, alpha=alpha, beta=beta, dtype=dtype)
+    if c_layout == mi.MI_C_COL_MAJOR:
+        C = np.ascontiguousarray(C.T)
+    if exact:
+        assert (C == ref).all(), f"{int((C != ref).sum())} elements differ"
+    rep = orc.check_tolerance(C, ref, K, orc.max_abs(A, dtype) * abs(alpha), orc.max_abs(B, dtype), dtype)
+    assert rep["violations"] == 0 and rep["compared"] == M * N, rep
+
+
+@pytest.mark.parametrize("config", all_configs(("tile", "ring", "mfma16", "ring16")))
+def test_alpha_beta_every_tiled_config_bit_exact_on_integer_fill(mi, orc, config):
+    # integer inputs, alpha a small integer or a power of two, beta a multiple of 1/4: acc * alpha
+    # and + beta are exact in fp32, so every summation order must give the oracle's bits
+    for (M, N, K), (alpha, beta) in [((512, 512, 512), (0.5, 3.0)), ((257, 515, 77), (-2.0, 0.25)),
+                                     ((300, 200, 136), (3.0, -1.5)), ((256, 384, 191), (1.0, 7.0)),
+                                     ((512, 768, 256), (0.25, 0.0))]:
+        check_epilogue(mi, orc, M, N, K, "int", alpha, beta, config=config, exact=True)
+
+
+@pytest.mark.parametrize("config", all_configs(("skinny", "stream")))
+def test_alpha_beta_decode_kernels(mi, orc, config):
+    from h100_gemm_amd import kernel_configs as kc
+    bm = kc.CONFIGS[config]["BM"]
+    for N, K in [(8192, 4096), (260, 192), (128, 64)]:      # several splits / one split
+        check_epilogue(mi, orc, bm - 1, N, K, "int", -0.5, 2.75, config=config, exact=True)
+    check_epilogue(mi, orc, bm, 2048, 8192, "normal", 0.37, 1.25, config=config)
+
+
+@pytest.mark.parametrize("M,N,K", [(512, 512, 512), (1024, 768, 256), (255, 511, 129), (16, 2048, 1024),
+                                   (64, 4096, 4096), (4095, 6143, 3073)])
+def test_alpha_beta_uniform_within_tolerance_auto_config(mi, orc, M, N, K):
+    check_epilogue(mi, orc, M, N, K, "uniform", 0.37, 1.25)
+    check_epilogue(mi, orc, M, N, K, "uniform", -1.5, 0.0)
+
+
+def test_alpha_one_beta_zero_is_the_plain_gemm(mi, orc):
+    for M, N, K in [(512, 512, 512), (257, 515, 77), (16, 2048, 1024), (100, 4096, 2048)]:
+        A, B = make_inputs(orc, M, N, K, "uniform")
+        d = Dev(mi, A, B, M, N)
+        plain = d.run(K)
+        assert (d.run_epilogue(K, 1.0, 0.0) == plain).all()
+
+
+@pytest.mark.parametrize("M,N,K", [(512, 512, 512), (257, 515, 77), (768, 256, 384), (16, 2048, 1024),
+                                   (2048, 16, 1024), (1, 7, 3)])
+def test_column_major_c_bit_exact_on_integer_fill(mi, orc, M, N, K):
+    check_epilogue(mi, orc, M, N, K, "int", 1.0, 0.0, c_layout=mi.MI_C_COL_MAJOR, exact=True)
+    check_epilogue(mi, orc, M, N, K, "int", 0.5, -3.0, c_layout=mi.MI_C_COL_MAJOR, exact=True)
+
+
+@pytest.mark.parametrize("M,N,K", [(1024, 768, 256), (4095, 6143, 3073), (128, 8192, 8192)])
+def test_column_major_c_uniform_within_tolerance(mi, orc, M, N, K):
+    check_epilogue(mi, orc, M, N, K, "uniform", 1.0, 0.0, c_layout=mi.MI_C_COL_MAJOR)
+
+
+def test_epilogue_fp16_and_argument_errors(mi, orc):
+    check_epilogue(mi, orc, 300, 200, 136, "int", 0.5, 1.0, dtype=1, exact=True)
+    check_epilogue(mi, orc, 300, 200, 136, "int", 0.5, 1.0, c_layout=mi.MI_C_COL_MAJOR, dtype=1, exact=True)
+    A, B = make_inputs(orc, 64, 64, 64, "int")
+    d = Dev(mi, A, B, 64, 64)
+    with pytest.raises(mi.MiGemmError, match="layout"):
+        d.run_epilogue(64, 1.0, 0.0, c_layout=2)
+    with pytest.raises(mi.MiGemmError, match="NaN"):
+        d.run_epilogue(64, float("nan"), 0.0)

@@ -68,6 +68,11 @@ def test_argument_validation_needs_no_device(mi):
     assert L.mi_gemm_ex(-1, 7, 8, 8, 8, 1, 1, 1, None, None) == mi._lib.MI_ERR_INVALID
     assert L.mi_gemm_ex(-1, bf, 70000, 70000, 8, 1, 1, 1, None, None) == mi._lib.MI_ERR_INVALID
     assert L.mi_reference_gpu_gemm(bf, 8, -1, 8, 1, 1, 1, 1.0, 0.0, None) == mi._lib.MI_ERR_INVALID
+    assert L.mi_gemm_epilogue(-1, bf, 8, 8, 8, 1, 1, 1, 1.0, 0.0, 2, None) == mi._lib.MI_ERR_INVALID
+    assert b"layout" in L.mi_last_error()
+    assert L.mi_gemm_epilogue(-1, bf, 8, 8, 8, 1, 1, 1, float("nan"), 0.0, 0, None) == mi._lib.MI_ERR_INVALID
+    assert L.mi_gemm_epilogue(-1, bf, 8, 0, 8, 1, 1, 1, 1.0, 0.0, mi.MI_C_COL_MAJOR, None) == mi._lib.MI_ERR_INVALID
+    assert L.mi_gemm_epilogue(-1, bf, 8, 8, 8, 1, None, 1, 1.0, 0.0, mi.MI_C_COL_MAJOR, None) == mi._lib.MI_ERR_INVALID
     with pytest.raises(mi.MiGemmError):
         mi.runKernel(8, 8, 0, 1, 1, 1)
     with pytest.raises(ValueError):
