@@ -349,6 +349,19 @@ void gpu_gemm(GemmParams<AType, BType, CType, AccumType> gemm_params, int config
                         nullptr));
 }
 
+// gpu_gemm with the epilogue the reference's kernels leave out: C = (CType)(acc * alpha + beta)
+// from the GemmParams (beta a plain scalar, reference.h:40), C row-major or column-major
+// (C[n*M + m], what the bf16 kernel behind runKernel writes, matmul_utils.cuh:529,545).
+template <class AType, class BType, class CType, class AccumType>
+void gpu_gemm_epilogue(GemmParams<AType, BType, CType, AccumType> gemm_params, int c_layout = MI_C_ROW_MAJOR,
+                       int config = MI_CONFIG_AUTO) {
+    static_assert(mi_dtype_of<AType>::value == mi_dtype_of<BType>::value &&
+                  mi_dtype_of<AType>::value == mi_dtype_of<CType>::value, "one storage type");
+    MI_CHECK(mi_gemm_epilogue(config, mi_dtype_of<AType>::value, gemm_params.M, gemm_params.N,
+                              gemm_params.K, gemm_params.A, gemm_params.B, gemm_params.C,
+                              (float)gemm_params.alpha, (float)gemm_params.beta, c_layout, nullptr));
+}
+
 // runKernel / run_kernel (matmul_h100_optimal.cu:32-59, 75-84).  kernel_num 1 is this
 // library's kernel.  0 is a vendor BLAS in the reference (runCublasGemmBF16,
 // matmul_h100_optimal.cu:63-73): the library links none, so a program that wants that arm

@@ -5,8 +5,14 @@
 #include "test_main.hpp"
 
 int main(int argc, char** argv) {
-    TestLaunchFn launch = [](int dtype, int config, int M, int N, int K, const void* A, const void* B,
-                             void* C) { MI_CHECK(mi_gemm_ex(config, dtype, M, N, K, A, B, C, nullptr, nullptr)); };
+    test_epilogue().supported = true;
+    TestLaunchFn launch = [](int dtype, int config, int M, int N, int K, const void* A, const void* B, void* C) {
+        const TestEpilogue& ep = test_epilogue();
+        if (ep.alpha == 1.0f && ep.beta == 0.0f && ep.c_layout == MI_C_ROW_MAJOR)
+            MI_CHECK(mi_gemm_ex(config, dtype, M, N, K, A, B, C, nullptr, nullptr));
+        else
+            MI_CHECK(mi_gemm_epilogue(config, dtype, M, N, K, A, B, C, ep.alpha, ep.beta, ep.c_layout, nullptr));
+    };
     auto label = [](int config) { return std::string(config == MI_CONFIG_AUTO ? "auto" : mi_gemm_config_name(config)); };
     auto parse = [](const char* value) {
         char* end = nullptr;

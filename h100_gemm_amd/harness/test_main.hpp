@@ -15,6 +15,11 @@
 //                        seeded U[-1,1), or seeded A ~ N(0,1), B ~ N(0,0.02^2); with the
 //                        last two the sums are inexact and the comparison is the bound
 //                        2^-7*|ref| + 1e-3*sqrt(K)*max|a|*max|b| instead of rtol
+//     alpha <a> beta <b> the golden's epilogue C = (CType)(acc*alpha + beta), beta a plain
+//                        scalar (reference.h:40; the reference's harness passes 1 and 0,
+//                        matmul_h100.cu.jinja:1014-1015)           } library build only:
+//     cmajor <0|1>       1: the kernel writes C column-major,      } the launch function
+//                        C[n*M + m] (matmul_utils.cuh:545)         } reads test_epilogue()
 #pragma once
 
 #include <functional>
@@ -24,6 +29,18 @@
 
 // launch(dtype, config, M, N, K, A, B, C): enqueue one GEMM on the null stream
 using TestLaunchFn = std::function<void(int, int, int, int, int, const void*, const void*, void*)>;
+
+// epilogue options of the run (alpha, beta, C layout); a launch function that cannot honour
+// them leaves `supported` false and test_main refuses non-default values
+struct TestEpilogue {
+    float alpha = 1.0f, beta = 0.0f;
+    int c_layout = MI_C_ROW_MAJOR;
+    bool supported = false;
+};
+inline TestEpilogue& test_epilogue() {
+    static TestEpilogue e;
+    return e;
+}
 
 const int testM = 4096;
 const int testN = 4096;
@@ -36,8 +53,9 @@ int run_test(int M, int N, int K, int config, int iters, bool check, const std::
     using BType = T;
     using CType = T;
     using AccumType = float;
-    AccumType alpha = 1.0;
-    AccumType beta = 0.0;
+    AccumType alpha = test_epilogue().alpha;
+    AccumType beta = test_epilogue().beta;
+    const bool cmajor = test_epilogue().c_layout == MI_C_COL_MAJOR;
     constexpr int dt = mi_dtype_of<T>::value;
 
     std::vector<int> AShape = {M, K};
@@ -79,6 +97,13 @@ int run_test(int M, int N, int K, int config, int iters, bool check, const std::
     }
     launch(dt, config, M, N, K, dA, dB, dC);
     copy_to_cpu(hC, dC, CShape);
+    if (cmajor) {   // bring the column-major result into the golden's row-major order
+        auto t = alloc_cpu_tensor<CType>(CShape);
+        for (int m = 0; m < M; ++m)
+            for (int n = 0; n < N; ++n) t[(size_t)m * N + n] = hC[(size_t)n * M + m];
+        free_cpu_tensor(hC);
+        hC = t;
+    }
     if (check) {
         if (fill == "int") {
             assert_allclose(hC, goldenC, CShape, /*rtol=*/1e-3, /*dump=*/false);
@@ -86,7 +111,7 @@ int run_test(int M, int N, int K, int config, int iters, bool check, const std::
             // inexact sums: a pure relative test fails on results near zero; use the bound
             // 2^-7*|ref| + 1e-3*sqrt(K)*max|a|*max|b| instead
             const size_t bad = verify_tolerance(goldenC, hC, shape_numel(CShape), K,
-                                                max_abs_value(hA, shape_numel(AShape)),
+                                                max_abs_value(hA, shape_numel(AShape)) * std::fabs((double)alpha),
                                                 max_abs_value(hB, shape_numel(BShape)));
             if (bad != 0) {
                 std::cout << "Wrong answer! " << bad << " errors!\n";
@@ -137,6 +162,9 @@ inline int test_main(int argc, char** argv, const TestLaunchFn& launch,
             else if (keys == "check") check = std::atoi(value) != 0;
             else if (keys == "dtype") dtype = value;
             else if (keys == "fill") fill = value;
+            else if (keys == "alpha") test_epilogue().alpha = (float)std::atof(value);
+            else if (keys == "beta") test_epilogue().beta = (float)std::atof(value);
+            else if (keys == "cmajor") test_epilogue().c_layout = std::atoi(value) ? MI_C_COL_MAJOR : MI_C_ROW_MAJOR;
             else if (keys == "cfg") {
                 config = parse_config(value);
                 if (config < 0) {
@@ -145,6 +173,11 @@ inline int test_main(int argc, char** argv, const TestLaunchFn& launch,
                 }
             }
         }
+    }
+    const TestEpilogue& ep = test_epilogue();
+    if (!ep.supported && (ep.alpha != 1.0f || ep.beta != 0.0f || ep.c_layout != MI_C_ROW_MAJOR)) {
+        std::cerr << "alpha / beta / cmajor need the library build of this program (gemm_test.cpp)\n";
+        return 2;
     }
     std::cout << "Shape M=" << M << ", N=" << N << ", K=" << K << "\n";
     if (dtype == "fp16") return run_test<half_t>(M, N, K, config, iters, check, fill, launch, label);

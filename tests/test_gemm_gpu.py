@@ -337,6 +337,10 @@ def test_harness_programs(mi):
     r = subprocess.run([str(h / "test"), "M", "333", "N", "129", "K", "77", "iters", "2",
                         "dtype", "fp16"], capture_output=True, text=True, timeout=120)
     assert r.returncode == 0 and "Correct!" in r.stdout, r.stdout + r.stderr
+    for extra in (["alpha", "0.5", "beta", "2"], ["cmajor", "1"], ["alpha", "-2", "beta", "0.25", "cmajor", "1", "fill", "uniform"]):
+        r = subprocess.run([str(h / "test"), "M", "333", "N", "129", "K", "77", "iters", "2", *extra],
+                           capture_output=True, text=True, timeout=120)
+        assert r.returncode == 0 and "Correct!" in r.stdout, r.stdout + r.stderr
     r = subprocess.run([str(h / "bf16_bench"), "1024", "4"], capture_output=True, text=True, timeout=120)
     assert r.returncode == 0, r.stdout + r.stderr
     assert "KERNEL 1" in r.stdout
