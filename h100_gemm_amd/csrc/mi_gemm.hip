@@ -49,19 +49,22 @@ bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 // Preconditions of the decode (split-K streaming) kernels: whole 16-byte chunks and whole
 // 64-deep K slabs, 8-byte aligned C rows.
 bool shape_is_streamable(int M, int N, int K, const void* A, const void* B, const void* C) {
-    return M <= 128 && N % 4 == 0 && K % 64 == 0 && aligned16(A) && aligned16(B) &&
+    (void)M;   // each decode kernel checks M against its own BM
+    return N % 4 == 0 && K % 64 == 0 && aligned16(A) && aligned16(B) &&
            (((uintptr_t)C & 7u) == 0);
 }
 
 // Split-K geometry for a decode launch.  These kernels are bound by memory latency, not by
 // CU count: about three quarters of the workgroups the chip can hold at once measured best
 // (8192 x 8192 weights, M = 64 and 128: 3 splits 30 / 38 us, 4 splits 35 / 41 us, 8 splits
-// 39 / 46 us).  At least four K slabs per split.  MI_GEMM_SPLITK=<n> overrides (tuning aid).
-int choose_splits(int tiles_n, int K, int cus, int lds_bytes) {
+// 39 / 46 us).  The 256-row kernel (one workgroup per CU, a single slab in flight) wants
+// every CU busy instead: M = 256, 2 / 3 / 4 / 6 splits run in 87 / 67 / 62 / 77 us.
+// At least four K slabs per split.  MI_GEMM_SPLITK=<n> overrides (tuning aid).
+int choose_splits(int tiles_n, int K, int cus, int lds_bytes, int bm) {
     static const int env = [] { const char* s = getenv("MI_GEMM_SPLITK"); return s ? atoi(s) : 0; }();
     const int slabs = K / 64;
     const int resident = cus * (lds_bytes > 0 && 160 * 1024 / lds_bytes > 1 ? 160 * 1024 / lds_bytes : 1);
-    int splits = env > 0 ? env : (3 * resident + 2 * tiles_n) / (4 * tiles_n);
+    int splits = env > 0 ? env : bm > 128 ? cus / tiles_n : (3 * resident + 2 * tiles_n) / (4 * tiles_n);
     if (splits > slabs / 4) splits = slabs / 4;
     if (splits < 1) splits = 1;
     if (splits > 64) splits = 64;
@@ -177,7 +180,7 @@ int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const vo
                         "config %s needs M <= %d, N %% 4 == 0, K %% 64 == 0 and 16-byte aligned operands",
                         e.name, e.BM);
         const int tiles_n = (N + e.BN - 1) / e.BN;
-        args.splits = choose_splits(tiles_n, K, compute_units(), e.lds_bytes);   // <= K / 64: no empty split
+        args.splits = choose_splits(tiles_n, K, compute_units(), e.lds_bytes, e.BM);   // <= K / 64: no empty split
         args.k_per_split = ((K / 64 + args.splits - 1) / args.splits) * 64;
         if (args.splits > 1) {
             hipError_t we = ensure_workspace((size_t)args.splits * M * N * sizeof(float), &args.ws);
@@ -242,7 +245,7 @@ int mi_gemm_config_grid(int config, int M, int N, int K) {
     if (e.kind == mi::KIND_SKINNY) {
         if (M > e.BM || K % 64 != 0) return 0;
         const int tiles_n = (N + e.BN - 1) / e.BN;
-        return tiles_n * choose_splits(tiles_n, K, compute_units(), e.lds_bytes);
+        return tiles_n * choose_splits(tiles_n, K, compute_units(), e.lds_bytes, e.BM);
     }
     return ((M + e.BM - 1) / e.BM) * ((N + e.BN - 1) / e.BN);
 }
@@ -250,7 +253,7 @@ int mi_gemm_config_grid(int config, int M, int N, int K) {
 int mi_gemm_select_config(int dtype, int M, int N, int K) {
     (void)dtype;
     // pointer alignment is unknown here: assume the usual 256-byte aligned allocations
-    return mi::select_kernel(M, N, K, M <= 128 && N % 4 == 0 && K % 64 == 0, compute_units());
+    return mi::select_kernel(M, N, K, N % 4 == 0 && K % 64 == 0, compute_units());
 }
 
 size_t mi_gemm_trace_words(int M, int N, int K) {

@@ -137,7 +137,13 @@ def test_config_table(mi):
     assert picked(4095, 6143, 3073) == (256, 192)
     assert picked(512, 512, 512) == (128, 128)
     assert kc.CONFIGS[mi.select_config(512, 512, 512)]['KIND'] == 'mfma16'
-    assert all("EFF" in kc.CONFIGS[mi.select_config(M, N, 4096)] for M in (129, 1000, 5000) for N in (100, 3000))
+    assert all("EFF" in kc.CONFIGS[mi.select_config(M, N, 4096)] for M in (257, 1000, 5000) for N in (100, 3000))
+    # 128 < M <= 256: the 256-row split-K kernel while the tiled kernels would leave CUs idle
+    assert mi.config_name(mi.select_config(129, 8192, 8192)) == "k256x128_n3"
+    assert mi.config_name(mi.select_config(256, 4096, 4096)) == "k256x128_n3"
+    assert "EFF" in kc.CONFIGS[mi.select_config(256, 28672, 8192)]       # many strips: tiled
+    assert "EFF" in kc.CONFIGS[mi.select_config(256, 8192, 1024)]        # short K: tiled
+    assert "EFF" in kc.CONFIGS[mi.select_config(200, 8190, 8192)]        # N % 4 != 0: tiled
     assert not kc.is_valid_config(dict(KIND="tile", BM=256, BN=256, WM=2, WN=2, SWZ=1, GROUP=8, OCC=2, DTL=0, EPI=0))
     assert not kc.is_valid_config(dict(KIND="tile", BM=96, BN=256, WM=2, WN=2, SWZ=1, GROUP=8, OCC=1, DTL=0, EPI=0))
     assert not kc.is_valid_config(dict(KIND="ring", BM=256, BN=256, WM=2, WN=2, NS=5, GROUP=8))
