@@ -83,7 +83,11 @@ __device__ __forceinline__ f32x4_t mfma_16x16x32(u32x4_t a, u32x4_t b, f32x4_t c
     }
 }
 
-template <class Cfg, bool TRACE = false>
+// SPLITK: the workgroup multiplies one piece of the K range of its tile (blockIdx.y) and
+// leaves an fp32 partial tile in the workspace instead of C.  A separate instantiation, so
+// that the plain kernel's registers and epilogue are untouched by it (a run-time branch to a
+// third epilogue made the 256-accumulator kernel spill in its last K step and epilogue).
+template <class Cfg, bool TRACE = false, bool SPLITK = false>
 __global__ void __launch_bounds__(Cfg::NT)
 __attribute__((amdgpu_waves_per_eu(Cfg::WAVES_PER_EU, Cfg::WAVES_PER_EU)))
 gemm_mfma16_kernel(const GemmArgs p) {
@@ -110,7 +114,12 @@ gemm_mfma16_kernel(const GemmArgs p) {
     tile_of_block<Cfg::GROUP>(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, tm, tn);
     const int row0 = tm * BM, col0 = tn * BN;
     constexpr bool EDGE = Cfg::EDGE;
-    const int M = p.M, N = p.N, K = p.K;
+    // Split-K: this workgroup multiplies the K range [k0, k0 + K) of its tile; k_per_split is a
+    // multiple of 128, so only the last piece can have a K tail.  Everything below works on
+    // the local range.
+    const int k0 = SPLITK ? (int)blockIdx.y * p.k_per_split : 0;
+    const int M = p.M, N = p.N;
+    const int K = SPLITK ? ((p.K - k0) < p.k_per_split ? (p.K - k0) : p.k_per_split) : p.K;
     // K steps: an even number.  The aligned variant is only launched with K % 128 == 0; the
     // predicated one rounds up and the surplus (part of a) slab is zeroed in LDS.
     const int KT = EDGE ? ((K + 2 * BK - 1) / (2 * BK)) * 2 : K / BK;
@@ -119,10 +128,14 @@ gemm_mfma16_kernel(const GemmArgs p) {
     // the end of a matrix is ever touched, and rows past M / N read as zeros.
     const int rowsA = (M - row0) < BM ? (M - row0) : BM;
     const int rowsB = (N - col0) < BN ? (N - col0) : BN;
-    const unsigned char* Ab = (const unsigned char*)p.A + (size_t)row0 * p.lda * 2;
-    const unsigned char* Bb = (const unsigned char*)p.B + (size_t)col0 * p.ldb * 2;
-    const uint32_t bytesA = (uint32_t)((rowsA - 1) * p.lda + K) * 2u;
-    const uint32_t bytesB = (uint32_t)((rowsB - 1) * p.ldb + K) * 2u;
+    const unsigned char* Ab = (const unsigned char*)p.A + ((size_t)row0 * p.lda + k0) * 2;
+    const unsigned char* Bb = (const unsigned char*)p.B + ((size_t)col0 * p.ldb + k0) * 2;
+    // (split-K: up to the true end of the last row, so that a piece that ends inside the row
+    // does not lose its last element to the dword-granular range check; K - k0 == K_local in
+    // the last piece, where the K-tail logic needs exactly that)
+    const int Kdesc = p.K - k0;
+    const uint32_t bytesA = (uint32_t)((rowsA - 1) * p.lda + Kdesc) * 2u;
+    const uint32_t bytesB = (uint32_t)((rowsB - 1) * p.ldb + Kdesc) * 2u;
     const __amdgpu_buffer_rsrc_t rsrcA = __builtin_amdgcn_make_buffer_rsrc((void*)Ab, 0, (int)bytesA, 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrcB = __builtin_amdgcn_make_buffer_rsrc((void*)Bb, 0, (int)bytesB, 0x00020000);
 
@@ -390,6 +403,27 @@ gemm_mfma16_kernel(const GemmArgs p) {
     unsigned char* Cb = (unsigned char*)p.C + (size_t)row0 * p.ldc * 2;
     const uint32_t bytesC = (uint32_t)(rowsA * p.ldc) * 2u;
     const __amdgpu_buffer_rsrc_t rsrcC = __builtin_amdgcn_make_buffer_rsrc((void*)Cb, 0, (int)bytesC, 0x00020000);
+    // split-K: fp32 partial tile -> ws[split][m][n], 16 bytes per lane straight from the
+    // accumulators (N % 4 == 0 is a launch precondition); splitk_reduce_kernel adds the
+    // splits in order, applies alpha / beta and rounds once
+    auto store_partials = [&]() __attribute__((always_inline)) {
+        // descriptor over this tile's rows of the split's M x N fp32 matrix: rows past M fall
+        // outside it and are dropped by the range check (the host keeps M*N*4 below 2^31)
+        float* P = p.ws + ((size_t)blockIdx.y * M + row0) * N;
+        const __amdgpu_buffer_rsrc_t rsrcP =
+            __builtin_amdgcn_make_buffer_rsrc((void*)P, 0, (int)((uint32_t)(rowsA * N) * 4u), 0x00020000);
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+            const int m_loc = wm * TM + i * 16 + l16;
+#pragma unroll
+            for (int j = 0; j < NI; ++j) {
+                const int n = col0 + wn * TN + j * 16 + 4 * q;
+                const uint32_t off = (uint32_t)(m_loc * N + n) * 4u;
+                if (!EDGE || n < N)
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, acc[i][j]), rsrcP, off, 0, 0);
+            }
+        }
+    };
     auto epilogue = [&](auto scaled_c) __attribute__((always_inline)) {
         // alpha / beta epilogue (see scale_acc): a second copy of this block behind a uniform branch
         constexpr bool SCALED = decltype(scaled_c)::value;
@@ -452,8 +486,12 @@ gemm_mfma16_kernel(const GemmArgs p) {
             }
         }
     };
-    if (p.alpha != 1.0f || p.beta != 0.0f) epilogue(std::true_type{});
-    else epilogue(std::false_type{});
+    if constexpr (SPLITK) {
+        store_partials();
+    } else {
+        if (p.alpha != 1.0f || p.beta != 0.0f) epilogue(std::true_type{});
+        else epilogue(std::false_type{});
+    }
     if constexpr (TRACE) {
         if (p.DB != nullptr && tid == 0) {
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -691,7 +729,12 @@ hipError_t launch_ring16_kernel(const GemmArgs& args, hipStream_t stream) {
 template <class Cfg, bool TRACE = false>
 hipError_t launch_mfma16_kernel(const GemmArgs& args, hipStream_t stream) {
     const int grid = args.tiles_m * args.tiles_n;
-    hipLaunchKernelGGL((gemm_mfma16_kernel<Cfg, TRACE>), dim3(grid), dim3(Cfg::NT), 0, stream, args);
+    if (args.splits > 1) {
+        if constexpr (TRACE) return hipErrorInvalidValue;   // no trace records from split-K launches
+        hipLaunchKernelGGL((gemm_mfma16_kernel<Cfg, false, true>), dim3(grid, args.splits), dim3(Cfg::NT), 0, stream, args);
+    } else {
+        hipLaunchKernelGGL((gemm_mfma16_kernel<Cfg, TRACE>), dim3(grid), dim3(Cfg::NT), 0, stream, args);
+    }
     return hipGetLastError();
 }
 

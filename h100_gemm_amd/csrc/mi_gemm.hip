@@ -17,6 +17,7 @@
 
 #include "../../include/mi_gemm.h"
 #include "gemm_kernel.hpp"
+#include "gemm_skinny_kernel.hpp"   // splitk_reduce_kernel
 #include "kernel_table.hpp"
 
 namespace mi {
@@ -69,6 +70,33 @@ int choose_splits(int tiles_n, int K, int cus, int lds_bytes, int bm) {
     if (splits < 1) splits = 1;
     if (splits > 64) splits = 64;
     return splits;
+}
+
+// Split-K for the tiled 16x16x32 kernel: when a shape has so few tiles that most CUs would
+// idle (small M x N, long K), the K range is cut into pieces of whole 128-deep steps, one
+// workgroup per (tile, piece); fp32 partials go to the workspace and splitk_reduce_kernel
+// adds them in order.  The piece count comes from the time model of the kernel table
+// (best_splits); the reduction's vector accesses need N % 4 == 0 and an 8-byte aligned C,
+// and a trace buffer has one record per tile, so those cases do not split.
+// MI_GEMM_TILE_SPLITK=<n> forces a piece count (1 = never split; tuning aid).
+bool shape_is_splittable(int N, const void* C, const int* DB) {
+    return DB == nullptr && N % 4 == 0 && ((uintptr_t)C & 7u) == 0;
+}
+
+int choose_tile_splits(const mi::KernelEntry& e, int M, int N, int K, bool splittable, int cus, int* k_per_split) {
+    *k_per_split = K;
+    static const int env = [] { const char* s = getenv("MI_GEMM_TILE_SPLITK"); return s ? atoi(s) : 0; }();
+    if (!splittable || e.kind != mi::KIND_MFMA16 || env == 1) return 1;
+    if (env > 1) {
+        int s = env < K / 512 ? env : K / 512;
+        if (s < 2 || (long long)((M + e.BM - 1) / e.BM) * ((N + e.BN - 1) / e.BN) * 256 * 256 * 4 >= 0x7fffffffLL) return 1;
+        const int kps = ((K + s - 1) / s + 127) / 128 * 128;
+        s = (K + kps - 1) / kps;
+        if (s < 2) return 1;
+        *k_per_split = kps;
+        return s;
+    }
+    return mi::best_splits(e, M, N, K, true, cus, k_per_split, nullptr);
 }
 
 // fp32 partial-sum workspace of the split-K kernels: one buffer per process, grown on
@@ -141,7 +169,8 @@ int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const vo
     int rc = check_args(config, dtype, M, N, K, A, B, C);
     if (rc != MI_OK) return rc;
     const bool streamable = shape_is_streamable(M, N, K, A, B, C);
-    if (config == MI_CONFIG_AUTO) config = mi::select_kernel(M, N, K, streamable, compute_units());
+    if (config == MI_CONFIG_AUTO)
+        config = mi::select_kernel(M, N, K, streamable, shape_is_splittable(N, C, DB), compute_units());
     const mi::KernelEntry& e = mi::kKernels[config];
 
     mi::GemmArgs args;
@@ -197,9 +226,30 @@ int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const vo
     mi::LaunchFn fn = e.launch[dtype][edge ? 1 : 0];
     if (!fn) return fail(MI_ERR_UNSUPPORTED, "config %s has no %s kernel for dtype %d", e.name,
                          edge ? "predicated" : "aligned", dtype);
+    if (e.kind == mi::KIND_MFMA16) {
+        args.splits = choose_tile_splits(e, M, N, K, shape_is_splittable(N, C, DB), compute_units(), &args.k_per_split);
+        if (args.splits > 1) {
+            hipError_t we = ensure_workspace((size_t)args.splits * M * N * sizeof(float), &args.ws);
+            if (we != hipSuccess)
+                return fail(MI_ERR_HIP, "split-K workspace allocation failed: %s", hipGetErrorString(we));
+        }
+    }
     hipError_t err = fn(args, (hipStream_t)stream);
     if (err != hipSuccess)
         return fail(MI_ERR_HIP, "launch of %s failed: %s", e.name, hipGetErrorString(err));
+    if (args.splits > 1) {
+        const size_t quads = ((size_t)M * N + 3) / 4;
+        const dim3 rgrid((unsigned)((quads + 255) / 256));
+        if (dtype == MI_DTYPE_BF16)
+            hipLaunchKernelGGL((mi::splitk_reduce_kernel<mi::DT_BF16>), rgrid, dim3(256), 0, (hipStream_t)stream,
+                               args.ws, C, M, N, N, args.splits, alpha, beta);
+        else
+            hipLaunchKernelGGL((mi::splitk_reduce_kernel<mi::DT_FP16>), rgrid, dim3(256), 0, (hipStream_t)stream,
+                               args.ws, C, M, N, N, args.splits, alpha, beta);
+        err = hipGetLastError();
+        if (err != hipSuccess)
+            return fail(MI_ERR_HIP, "launch of the split-K reduction failed: %s", hipGetErrorString(err));
+    }
     return MI_OK;
 }
 
@@ -247,13 +297,18 @@ int mi_gemm_config_grid(int config, int M, int N, int K) {
         const int tiles_n = (N + e.BN - 1) / e.BN;
         return tiles_n * choose_splits(tiles_n, K, compute_units(), e.lds_bytes, e.BM);
     }
-    return ((M + e.BM - 1) / e.BM) * ((N + e.BN - 1) / e.BN);
+    const int tiles = ((M + e.BM - 1) / e.BM) * ((N + e.BN - 1) / e.BN);
+    if (e.kind == mi::KIND_MFMA16) {   // split-K pieces, assuming an aligned C and no trace buffer
+        int kps = K;
+        return tiles * choose_tile_splits(e, M, N, K, N % 4 == 0, compute_units(), &kps);
+    }
+    return tiles;
 }
 
 int mi_gemm_select_config(int dtype, int M, int N, int K) {
     (void)dtype;
     // pointer alignment is unknown here: assume the usual 256-byte aligned allocations
-    return mi::select_kernel(M, N, K, N % 4 == 0 && K % 64 == 0, compute_units());
+    return mi::select_kernel(M, N, K, N % 4 == 0 && K % 64 == 0, N % 4 == 0, compute_units());
 }
 
 size_t mi_gemm_trace_words(int M, int N, int K) {

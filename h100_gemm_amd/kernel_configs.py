@@ -209,7 +209,6 @@ CONFIGS = [
     _k(32, NS=4),
     _k(64, NS=6),
     _k(128, NS=5),
-    _k(256, NS=3),
 ]
 
 assert all(is_valid_config(c) for c in CONFIGS), [config_name(c) for c in CONFIGS if not is_valid_config(c)]
@@ -224,11 +223,9 @@ assert all(n in {config_name(c) for c in CONFIGS} for n in TUNED_SHAPES.values()
 # Automatic choice for decode shapes (the kernels' preconditions permitting): (largest M,
 # config name, largest N per compute unit or 0 for any, smallest K), first match wins.
 # Up to M = 32 the single-pass kernel; above, the split-K kernel measured ahead of it
-# (M = 64: 30 us against 33 us).  128 < M <= 256 takes the split-K kernel while the tiled
-# kernels would leave half the CUs idle (N <= 8192 on 256 CUs: 128 tiles of 128 x 128) and K
-# is long enough for four or more splits: M = 256, K = 8192, N = 1024 / 4096 / 8192 run in
-# 30 / 36 / 62 us against 59 / 56 / 96 us tiled; K = 4096: 21 / 28 / 35 against 30 / 32 / 34;
-# at K = 1024 or N >= 16384 the tiled kernels are ahead (N = 28672: 147 us against 189 us).
+# (M = 64: 30 us against 33 us).  Above M = 128 the tiled kernels with split-K take over
+# (256 x 8192 x 8192: 48.8 us as 256x128 tiles x 4 pieces; a 256-row variant of the decode
+# kernel, one slab in flight per CU, took 61 us and was dropped).
 DECODE_LADDER = [(16, "s16x32_n5", 0, 0), (32, "s32x32_n4", 0, 0), (64, "k64x128_n6", 0, 0),
-                 (128, "k128x128_n5", 0, 0), (256, "k256x128_n3", 32, 4096)]
+                 (128, "k128x128_n5", 0, 0)]
 assert all(n in {config_name(c) for c in CONFIGS} for _, n, _, _ in DECODE_LADDER)

@@ -435,3 +435,38 @@ def test_epilogue_fp16_and_argument_errors(mi, orc):
         d.run_epilogue(64, 1.0, 0.0, c_layout=2)
     with pytest.raises(mi.MiGemmError, match="NaN"):
         d.run_epilogue(64, float("nan"), 0.0)
+
+
+# ------------------------------------------- split-K of the tiled 16x16x32 kernel ----------
+
+@pytest.mark.parametrize("config", all_configs(("mfma16",)))
+def test_tiled_split_k_bit_exact_on_integer_fill(mi, orc, config):
+    """Few tiles and a long K: the K range is cut into pieces, fp32 partials are added in order.
+    Integer fills keep every partial sum exact, so the result must match the oracle's bits."""
+    from h100_gemm_amd import kernel_configs as kc
+    c = kc.CONFIGS[config]
+    for M, N, K in [(512, 768, 4096), (300, 260, 5000), (256, 256, 8192 + 64), (130, 512, 2048)]:
+        tiles = -(-M // c["BM"]) * -(-N // c["BN"])
+        assert mi.config_grid(config, M, N, K) >= 2 * tiles, "shape chosen so that split-K is in effect"
+        check(mi, orc, M, N, K, "int", config=config, exact=True)
+
+
+def test_tiled_split_k_auto_config_uniform_fp16_and_epilogue(mi, orc):
+    for M, N, K in [(512, 512, 4096), (512, 512, 8192), (1000, 500, 3000)]:
+        cfg = mi.select_config(M, N, K)
+        assert mi.config_grid(cfg, M, N, K) > -(-M // 128) * -(-N // 128) or "mfma16" not in str(cfg)
+        check(mi, orc, M, N, K, "uniform")
+    check(mi, orc, 512, 512, 4096, "int", dtype=1, exact=True)
+    check_epilogue(mi, orc, 512, 512, 4096, "int", 0.5, -3.0, exact=True)
+    check_epilogue(mi, orc, 300, 260, 5000, "uniform", 0.37, 1.25)
+    check_epilogue(mi, orc, 4096, 256, 4096, "int", 2.0, 1.0, c_layout=mi.MI_C_COL_MAJOR, exact=True)
+    # odd N: no split-K (the reduction needs N % 4 == 0), same answer
+    check(mi, orc, 512, 511, 4096, "int", exact=True)
+
+
+def test_tiled_split_k_is_deterministic(mi, orc):
+    A, B = make_inputs(orc, 512, 512, 8192, "uniform")
+    d = Dev(mi, A, B, 512, 512)
+    first = d.run(8192)
+    for _ in range(3):
+        assert (d.run(8192) == first).all()

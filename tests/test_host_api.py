@@ -138,11 +138,16 @@ def test_config_table(mi):
     assert picked(512, 512, 512) == (128, 128)
     assert kc.CONFIGS[mi.select_config(512, 512, 512)]['KIND'] == 'mfma16'
     assert all("EFF" in kc.CONFIGS[mi.select_config(M, N, 4096)] for M in (257, 1000, 5000) for N in (100, 3000))
-    # 128 < M <= 256: the 256-row split-K kernel while the tiled kernels would leave CUs idle
-    assert mi.config_name(mi.select_config(129, 8192, 8192)) == "k256x128_n3"
-    assert mi.config_name(mi.select_config(256, 4096, 4096)) == "k256x128_n3"
-    assert "EFF" in kc.CONFIGS[mi.select_config(256, 28672, 8192)]       # many strips: tiled
-    assert "EFF" in kc.CONFIGS[mi.select_config(256, 8192, 1024)]        # short K: tiled
+    # few tiles and a long K: split-K pieces of a tiled kernel fill the CUs
+    c = mi.select_config(256, 8192, 8192)
+    assert kc.CONFIGS[c]["KIND"] == "mfma16" and (kc.CONFIGS[c]["BM"], kc.CONFIGS[c]["BN"]) == (256, 128)
+    assert 128 < mi.config_grid(c, 256, 8192, 8192) <= 256          # 64 tiles x 3 or 4 pieces
+    c = mi.select_config(512, 512, 4096)
+    assert mi.config_grid(c, 512, 512, 4096) == 16 * 8              # 128x128 tiles x 8 pieces of 512
+    assert mi.config_grid(mi.select_config(8192, 8192, 8192), 8192, 8192, 8192) == 1024   # no split-K when the tiles fill the chip
+    assert mi.config_grid(mi.select_config(512, 512, 512), 512, 512, 512) == 16           # nor for a short K
+    c = mi.select_config(512, 510, 4096)
+    assert mi.config_grid(c, 512, 510, 4096) == -(-512 // kc.CONFIGS[c]["BM"]) * -(-510 // kc.CONFIGS[c]["BN"])   # N % 4 != 0: no split-K
     assert "EFF" in kc.CONFIGS[mi.select_config(200, 8190, 8192)]        # N % 4 != 0: tiled
     assert not kc.is_valid_config(dict(KIND="tile", BM=256, BN=256, WM=2, WN=2, SWZ=1, GROUP=8, OCC=2, DTL=0, EPI=0))
     assert not kc.is_valid_config(dict(KIND="tile", BM=96, BN=256, WM=2, WN=2, SWZ=1, GROUP=8, OCC=1, DTL=0, EPI=0))

@@ -76,7 +76,7 @@ def test_aligned_kernels_do_not_spill(asm_text):
         found = re.findall(r"\.amdhsa_kernel (\S+).*?\.amdhsa_private_segment_fixed_size (\d+)", text, flags=re.S)
         assert found, unit
         # Mfma16Config<..., EDGE, OCC>, TRACE: "...ELb<EDGE>ELi<OCC>EEELb<TRACE>EE..."
-        aligned = [(n, int(sz)) for n, sz in found if re.search(r"Mfma16ConfigI\w*?ELb0ELi\d+EEELb[01]E", n)]
+        aligned = [(n, int(sz)) for n, sz in found if re.search(r"Mfma16ConfigI\w*?ELb0ELi\d+EEELb[01]ELb[01]E", n)]
         assert aligned, (unit, [n for n, _ in found])
         for n, sz in aligned:
             assert sz == 0, f"{unit}: {n} uses {sz} bytes of scratch per lane"
