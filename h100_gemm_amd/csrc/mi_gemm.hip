@@ -83,7 +83,8 @@ bool shape_is_splittable(int N, const void* C, const int* DB) {
     return DB == nullptr && N % 4 == 0 && ((uintptr_t)C & 7u) == 0;
 }
 
-int choose_tile_splits(const mi::KernelEntry& e, int M, int N, int K, bool splittable, int cus, int* k_per_split) {
+int choose_tile_splits(const mi::KernelEntry& e, int M, int N, int K, bool splittable, bool ptr_aligned, int cus,
+                       int* k_per_split) {
     *k_per_split = K;
     static const int env = [] { const char* s = getenv("MI_GEMM_TILE_SPLITK"); return s ? atoi(s) : 0; }();
     if (!splittable || e.kind != mi::KIND_MFMA16 || env == 1) return 1;
@@ -96,7 +97,7 @@ int choose_tile_splits(const mi::KernelEntry& e, int M, int N, int K, bool split
         *k_per_split = kps;
         return s;
     }
-    return mi::best_splits(e, M, N, K, true, cus, k_per_split, nullptr);
+    return mi::best_splits(e, M, N, K, true, ptr_aligned, cus, k_per_split, nullptr);
 }
 
 // fp32 partial-sum workspace of the split-K kernels: one buffer per process, grown on
@@ -170,7 +171,8 @@ int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const vo
     if (rc != MI_OK) return rc;
     const bool streamable = shape_is_streamable(M, N, K, A, B, C);
     if (config == MI_CONFIG_AUTO)
-        config = mi::select_kernel(M, N, K, streamable, shape_is_splittable(N, C, DB), compute_units());
+        config = mi::select_kernel(M, N, K, streamable, shape_is_splittable(N, C, DB),
+                                   aligned16(A) && aligned16(B) && aligned16(C), compute_units());
     const mi::KernelEntry& e = mi::kKernels[config];
 
     mi::GemmArgs args;
@@ -227,7 +229,8 @@ int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const vo
     if (!fn) return fail(MI_ERR_UNSUPPORTED, "config %s has no %s kernel for dtype %d", e.name,
                          edge ? "predicated" : "aligned", dtype);
     if (e.kind == mi::KIND_MFMA16) {
-        args.splits = choose_tile_splits(e, M, N, K, shape_is_splittable(N, C, DB), compute_units(), &args.k_per_split);
+        args.splits = choose_tile_splits(e, M, N, K, shape_is_splittable(N, C, DB),
+                                         aligned16(A) && aligned16(B) && aligned16(C), compute_units(), &args.k_per_split);
         if (args.splits > 1) {
             hipError_t we = ensure_workspace((size_t)args.splits * M * N * sizeof(float), &args.ws);
             if (we != hipSuccess)
@@ -300,7 +303,7 @@ int mi_gemm_config_grid(int config, int M, int N, int K) {
     const int tiles = ((M + e.BM - 1) / e.BM) * ((N + e.BN - 1) / e.BN);
     if (e.kind == mi::KIND_MFMA16) {   // split-K pieces, assuming an aligned C and no trace buffer
         int kps = K;
-        return tiles * choose_tile_splits(e, M, N, K, N % 4 == 0, compute_units(), &kps);
+        return tiles * choose_tile_splits(e, M, N, K, N % 4 == 0, true, compute_units(), &kps);
     }
     return tiles;
 }
@@ -308,7 +311,7 @@ int mi_gemm_config_grid(int config, int M, int N, int K) {
 int mi_gemm_select_config(int dtype, int M, int N, int K) {
     (void)dtype;
     // pointer alignment is unknown here: assume the usual 256-byte aligned allocations
-    return mi::select_kernel(M, N, K, N % 4 == 0 && K % 64 == 0, N % 4 == 0, compute_units());
+    return mi::select_kernel(M, N, K, N % 4 == 0 && K % 64 == 0, N % 4 == 0, true, compute_units());
 }
 
 size_t mi_gemm_trace_words(int M, int N, int K) {

@@ -23,6 +23,8 @@ template takes (matmul_h100.cu.jinja:9-14) -- re-cast for CDNA4:
              register-staged predicated kernel runs best with eight waves)
     EFF      (optional) per-CU throughput relative to the 256x256 tile, measured at 8192^3;
              configs that carry it are the candidates of the automatic shape -> kernel choice
+    EFF_E    (optional) throughput of the predicated variant relative to the aligned one, from
+             7000^3, 6000^3 and 5000^3 (default 0.85); used for shapes the aligned variant cannot run
 
 The index of a config in ``CONFIGS`` is its ``config`` number in the C ABI.
 """
@@ -154,8 +156,10 @@ def _r(BM, BN, WM, WN, NS=4, GROUP=8):
     return dict(KIND="ring", BM=BM, BN=BN, WM=WM, WN=WN, NS=NS, GROUP=GROUP)
 
 
-def _m(BM, BN, WM, WN, GROUP=4, EFF=None, DRAIN=0, OCC=1):
+def _m(BM, BN, WM, WN, GROUP=4, EFF=None, DRAIN=0, OCC=1, EFF_E=None):
     c = dict(KIND="mfma16", BM=BM, BN=BN, WM=WM, WN=WN, GROUP=GROUP)
+    if EFF_E is not None:
+        c["EFF_E"] = EFF_E
     if OCC != 1:
         c["OCC"] = OCC
     if DRAIN:
@@ -193,11 +197,11 @@ CONFIGS = [
     _r(256, 256, 2, 2),
     _r(256, 256, 2, 4),
     _m(256, 256, 2, 2),
-    _m(256, 256, 2, 2, DRAIN=3, EFF=1.0),
-    _m(256, 192, 2, 2, DRAIN=3, EFF=0.89),
-    _m(128, 256, 2, 2, DRAIN=1, EFF=0.875),
-    _m(256, 128, 2, 2, DRAIN=1, EFF=0.845),
-    _m(128, 128, 2, 2, DRAIN=1, OCC=2, EFF=0.78),
+    _m(256, 256, 2, 2, DRAIN=3, EFF=1.0, EFF_E=0.82),
+    _m(256, 192, 2, 2, DRAIN=3, EFF=0.89, EFF_E=0.90),
+    _m(128, 256, 2, 2, DRAIN=1, EFF=0.875, EFF_E=0.80),
+    _m(256, 128, 2, 2, DRAIN=1, EFF=0.845, EFF_E=0.80),
+    _m(128, 128, 2, 2, DRAIN=1, OCC=2, EFF=0.78, EFF_E=0.74),
     _m(256, 256, 4, 2),
     _m(256, 256, 4, 2, DRAIN=3),
     _m(256, 256, 2, 4),
@@ -209,6 +213,8 @@ CONFIGS = [
     _k(32, NS=4),
     _k(64, NS=6),
     _k(128, NS=5),
+    _m(192, 192, 2, 2, DRAIN=1, EFF=0.80, EFF_E=0.91),
+    _m(192, 128, 2, 2, DRAIN=1, EFF=0.74, EFF_E=0.85),
 ]
 
 assert all(is_valid_config(c) for c in CONFIGS), [config_name(c) for c in CONFIGS if not is_valid_config(c)]
