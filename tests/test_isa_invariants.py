@@ -9,23 +9,30 @@ import pytest
 
 ROOT = Path(__file__).resolve().parent.parent
 GEN = ROOT / "h100_gemm_amd" / "csrc" / "gen"
-UNITS = ["unit_m256x256_w2x2_g4_b3.hip", "unit_m256x192_w2x2_g4_b3.hip"]
+def mfma16_units():
+    from h100_gemm_amd import kernel_configs as kc
+    return [f"unit_{kc.config_name(c)}.hip" for c in kc.CONFIGS if c["KIND"] == "mfma16"]
 
 
 @pytest.fixture(scope="module")
 def asm_text(tmp_path_factory):
+    """assembly text of every 16x16x32-kernel unit (all of them keep M0 live across asm statements)"""
+    from concurrent.futures import ThreadPoolExecutor
     from h100_gemm_amd import build
     build.render_sources()
-    out = {}
-    for unit in UNITS:
+    tmp = tmp_path_factory.mktemp("isa")
+
+    def one(unit):
         src = GEN / unit
         assert src.exists(), src
-        dst = tmp_path_factory.mktemp("isa") / (src.stem + ".s")
+        dst = tmp / (src.stem + ".s")
         cmd = ["/opt/rocm/bin/hipcc", *build.HIPFLAGS, "--cuda-device-only", "-S", f"-I{build.CSRC}", f"-I{GEN}",
                str(src), "-o", str(dst)]
-        subprocess.run(cmd, check=True, capture_output=True, timeout=600)
-        out[unit] = dst.read_text()
-    return out
+        subprocess.run(cmd, check=True, capture_output=True, timeout=900)
+        return unit, dst.read_text()
+
+    with ThreadPoolExecutor(8) as ex:
+        return dict(ex.map(one, mfma16_units()))
 
 
 def kernels(text):
@@ -42,7 +49,7 @@ def test_m0_is_only_written_by_the_kernels_own_asm(asm_text):
     directly is preceded by the wait state the hardware needs."""
     for unit, text in asm_text.items():
         ks = kernels(text)
-        assert len(ks) >= 4, (unit, list(ks))
+        assert len(ks) >= 8, (unit, list(ks))      # {bf16, fp16} x {aligned, predicated} x {plain, trace, split-K}
         for name, body in ks.items():
             inasm, prev = False, ""
             loads = sets = 0
@@ -69,9 +76,16 @@ def test_m0_is_only_written_by_the_kernels_own_asm(asm_text):
 
 
 def test_aligned_kernels_do_not_spill(asm_text):
-    """The 256 accumulators live in AGPRs and the aligned variants keep everything else in
-    VGPRs: no scratch memory (the predicated variants spill in their peeled tail only)."""
+    """The accumulators live in AGPRs and the aligned variants keep everything else in VGPRs:
+    no scratch memory (the predicated variants spill in their peeled tail only).  Checked for
+    the candidates of the automatic choice (the eight-wave tuner variants have half the
+    registers per wave and may spill a few)."""
+    from h100_gemm_amd import kernel_configs as kc
+    auto = {f"unit_{kc.config_name(c)}.hip" for c in kc.CONFIGS if c["KIND"] == "mfma16" and c.get("EFF")}
+    assert len(auto) >= 5
     for unit, text in asm_text.items():
+        if unit not in auto:
+            continue
         # kernel descriptors: ".amdhsa_kernel NAME ... .amdhsa_private_segment_fixed_size N"
         found = re.findall(r"\.amdhsa_kernel (\S+).*?\.amdhsa_private_segment_fixed_size (\d+)", text, flags=re.S)
         assert found, unit
