@@ -470,3 +470,24 @@ def test_tiled_split_k_is_deterministic(mi, orc):
     first = d.run(8192)
     for _ in range(3):
         assert (d.run(8192) == first).all()
+
+
+def test_tiled_split_k_random_shapes_and_alignments(mi, orc):
+    # seeded sweep over few-tile shapes with a long, ragged K (split-K pieces with a K tail in
+    # the last one), operands at arbitrary even byte offsets; C at 8-byte offsets (split-K) and at
+    # 2-byte offsets (the reduction cannot be used: one piece); automatic choice and every
+    # candidate tile of it
+    from h100_gemm_amd import kernel_configs as kc
+    rng = np.random.default_rng(20241125)
+    configs = [-1] + [i for i, c in enumerate(kc.CONFIGS) if c["KIND"] == "mfma16" and c.get("EFF")]
+    for it in range(32):
+        M = int(rng.integers(1, 420))
+        N = int(rng.integers(1, 110)) * 4
+        K = int(rng.choice([rng.integers(2048, 6000), 128 * rng.integers(16, 40), 128 * rng.integers(16, 40) + rng.integers(1, 9)]))
+        offA, offB = (int(2 * rng.integers(0, 16)) for _ in range(2))
+        offC = int(rng.choice([0, 8, 16, 2, 6]))
+        config = configs[it % len(configs)]
+        print(f"case {it}: M={M} N={N} K={K} offsets {offA},{offB},{offC} config={config}", flush=True)
+        C, ref, guard = _run_offset(mi, orc, config, M, N, K, offA, offB, offC)
+        assert (C == ref).all(), f"{int((C != ref).sum())} elements differ"
+        assert (guard == 0xEEEE).all(), "bytes outside C were written"
