@@ -72,7 +72,7 @@ class GemmTuner:
         # Define parameter search space
         self.param_space = {
             'KIND': ['mfma16', 'ring', 'ring16', 'tile'],
-            'BM': [128, 256],
+            'BM': [128, 192, 256],
             'BN': [128, 192, 256],
             'WM': [2, 4],
             'WN': [2, 4],
