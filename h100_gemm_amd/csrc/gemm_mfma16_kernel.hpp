@@ -279,7 +279,12 @@ gemm_mfma16_kernel(const GemmArgs p) {
             for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.0f;
 
     auto mma_one = [&](int buf, int idx) __attribute__((always_inline)) {
-        const int i = idx / NI, j = idx % NI;
+        // rows of accumulator tiles in turn, columns back and forth: srcB (the A fragment) stays
+        // for a whole row and srcA (the B fragment) is kept across the turn, so every MFMA
+        // changes one operand only.  The chip is power limited and operand changes cost power:
+        // same cycle count, 0.3-1 % less time than always starting a row at column 0 (and the
+        // column-major order, srcB changing every time, measured 8 % slower).
+        const int i = idx / NI, j = (i & 1) ? NI - 1 - idx % NI : idx % NI;
         acc[i][j] = mfma_16x16x32<DT>(fb[buf][j], fa[buf][i], acc[i][j]);
     };
     // fragment r of a slice in the order the MFMAs first need them: A0, B0..B(NI-1), A1..
