@@ -48,7 +48,7 @@ WORKLOADS = {
 # FETCH_SIZE counts KiB and reads half of what a plain 256 MiB device copy moves (131087 for
 # 262144 KiB read), so it is scaled by 2.0; WRITE_SIZE reads the copy's writes exactly (1.0).
 MEASURED_TRAFFIC_BYTES = {
-    "square8192": (786789 * 2.0 + 131078) * 1024,     # 1.75 GB against 0.40 GB algorithmic
+    "square8192": (787026 * 2.0 + 131083) * 1024,     # 1.75 GB against 0.40 GB algorithmic
     "skinny16": (66589.6 * 2.0 + 256) * 1024,         # 0.137 GB: B is read exactly once
     "unaligned": (130105 * 2.0 + 49737) * 1024,       # 0.317 GB against 0.113 GB algorithmic
     "mlp_down": (2.7535e6 * 2.0 + 131072) * 1024,      # 5.8 GB against 1.07 GB algorithmic
