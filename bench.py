@@ -105,7 +105,7 @@ def main() -> int:
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
-              "(the GEMM shards by splitting N or M across GPUs with no exchange; see DESIGN.md)",
+              "(the GEMM shards by splitting N or M across GPUs with no exchange, each GPU running this kernel on its part)",
               file=sys.stderr)
         return 2
     if int(os.environ.get("WORLD_SIZE", "1")) != 1:
