@@ -40,6 +40,27 @@ def test_library_links_no_vendor_blas(mi):
     assert not [n for n in needed if re.search(r"blas|tensile|miopen|torch", n, re.I)], needed
 
 
+def test_header_is_plain_c_and_links(mi, tmp_path):
+    """include/mi_gemm.h is a C header (what a cgo / JNI / ctypes binding would consume): a C99
+    program that takes the address of every declared function compiles with -pedantic -Werror,
+    links against the library and runs (no device call is made)."""
+    from h100_gemm_amd import _lib
+    names = declared_functions()
+    src = tmp_path / "abi.c"
+    src.write_text('#include "include/mi_gemm.h"\n#include <stdio.h>\ntypedef void (*fn)(void);\n'
+                   + "static fn table[] = {" + ", ".join(f"(fn){n}" for n in names) + "};\n"
+                   + 'int main(void) {\n    if (sizeof table / sizeof table[0] < 20 || !table[0]) return 1;\n'
+                   + '    if (mi_gemm_bf16(0, 1, 1, 0, 0, 0, 0, 0) != MI_ERR_INVALID) return 2;\n'
+                   + '    puts(mi_last_error());\n    return mi_gemm_num_configs() > 0 ? 0 : 3;\n}\n')
+    exe = tmp_path / "abi"
+    libdir = _lib.LIB_PATH.parent
+    r = subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Werror", "-Wno-pedantic", f"-I{ROOT}", str(src), "-o", str(exe),
+                        f"-L{libdir}", "-lmi_gemm", f"-Wl,-rpath,{libdir}"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    r = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert r.returncode == 0 and "positive" in r.stdout, r.stdout + r.stderr
+
+
 def test_missing_library_fails_loudly(mi, monkeypatch, tmp_path):
     from h100_gemm_amd import _lib
     monkeypatch.setattr(_lib, "_lib", None)
