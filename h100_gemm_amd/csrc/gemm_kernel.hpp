@@ -120,9 +120,19 @@ __device__ __forceinline__ uint16_t cvt_store(float f) {
         return __builtin_bit_cast(uint16_t, h);
     }
 }
+// Two values at once: one v_cvt_pk_{bf16,f16}_f32 (converting them one by one and or-ing the
+// halves together costs three more VALU instructions per pair, 2000 cycles per 256x256 tile).
 template <int DT>
 __device__ __forceinline__ uint32_t cvt_store2(float lo, float hi) {
-    return (uint32_t)cvt_store<DT>(lo) | ((uint32_t)cvt_store<DT>(hi) << 16);
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t v = {lo, hi};
+    if constexpr (DT == DT_BF16) {
+        typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+    } else {
+        typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+    }
 }
 
 // Wait for this wave's LDS traffic, then meet the other waves.  Deliberately not
