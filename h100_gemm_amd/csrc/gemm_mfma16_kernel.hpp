@@ -303,6 +303,12 @@ gemm_mfma16_kernel(const GemmArgs p) {
     for (int d = 0; d < LA + LB; ++d) dma_one(0, 0, d);
 #pragma unroll
     for (int d = 0; d < LA + LB; ++d) dma_one(1, 1, d);
+    // Pin the zeroing of the accumulators here, while the first slabs are on their way: left
+    // alone, the compiler zeroes every accumulator register twice, after the wait for slab 0.
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) asm volatile("" : "+a"(acc[i][j]));
     if constexpr (EDGE) {
         asm volatile("s_waitcnt vmcnt(%0)" :: "n"(LA + LB) : "memory");            // own loads of slab 0 are in
         if (BK > K) fix_tail(0, 0);
