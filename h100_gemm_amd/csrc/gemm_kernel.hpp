@@ -147,9 +147,17 @@ __device__ __forceinline__ void lds_barrier() {
 // what SCALED = false leaves out entirely: the kernels hold two copies of their epilogue
 // behind one uniform branch, so the unscaled path and the K loop are unchanged by it.
 // (Scaling the accumulators in place before a single epilogue costs registers in the loop.)
+// x * a + b as two separately rounded fp32 operations.  (HIP's __fmul_rn / __fadd_rn are the
+// plain operators and are contracted into one v_fma_f32 under the default -ffp-contract=fast;
+// without the `contract` flag on these two operations they cannot be.)
+__device__ __forceinline__ float mul_add_unfused(float x, float a, float b) {
+#pragma clang fp contract(off)
+    const float t = x * a;
+    return t + b;
+}
 template <bool SCALED>
 __device__ __forceinline__ float scale_acc(float x, float alpha, float beta) {
-    if constexpr (SCALED) return __fadd_rn(__fmul_rn(x, alpha), beta);
+    if constexpr (SCALED) return mul_add_unfused(x, alpha, beta);
     else return x;
 }
 

@@ -276,10 +276,10 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restr
         a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
     }
     if (alpha != 1.0f || beta != 0.0f) {
-        a.x = __fadd_rn(__fmul_rn(a.x, alpha), beta);
-        a.y = __fadd_rn(__fmul_rn(a.y, alpha), beta);
-        a.z = __fadd_rn(__fmul_rn(a.z, alpha), beta);
-        a.w = __fadd_rn(__fmul_rn(a.w, alpha), beta);
+        a.x = mul_add_unfused(a.x, alpha, beta);
+        a.y = mul_add_unfused(a.y, alpha, beta);
+        a.z = mul_add_unfused(a.z, alpha, beta);
+        a.w = mul_add_unfused(a.w, alpha, beta);
     }
     const size_t m = idx / N, n = idx % N;
     u32x2_t w;

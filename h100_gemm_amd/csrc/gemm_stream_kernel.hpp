@@ -167,10 +167,10 @@ __global__ void __launch_bounds__(256) gemm_stream_kernel(const SkinnyArgs p) {
             sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
         }
         if (p.alpha != 1.0f || p.beta != 0.0f) {
-            sum.x = __fadd_rn(__fmul_rn(sum.x, p.alpha), p.beta);
-            sum.y = __fadd_rn(__fmul_rn(sum.y, p.alpha), p.beta);
-            sum.z = __fadd_rn(__fmul_rn(sum.z, p.alpha), p.beta);
-            sum.w = __fadd_rn(__fmul_rn(sum.w, p.alpha), p.beta);
+            sum.x = mul_add_unfused(sum.x, p.alpha, p.beta);
+            sum.y = mul_add_unfused(sum.y, p.alpha, p.beta);
+            sum.z = mul_add_unfused(sum.z, p.alpha, p.beta);
+            sum.w = mul_add_unfused(sum.w, p.alpha, p.beta);
         }
         if (m < M && col0 + n < N) {                         // N % 4 == 0 is a launch precondition
             u32x2_t w2;

@@ -24,6 +24,13 @@ __device__ __forceinline__ float load_f32(const uint16_t* p) {
         return (float)__builtin_bit_cast(_Float16, *p);
     }
 }
+// x * a + b as two separately rounded fp32 operations (HIP's __fmul_rn / __fadd_rn are the
+// plain operators and would be contracted into one fma under the default -ffp-contract=fast)
+__device__ __forceinline__ float mul_add_unfused(float x, float a, float b) {
+#pragma clang fp contract(off)
+    const float t = x * a;
+    return t + b;
+}
 template <int DT>
 __device__ __forceinline__ uint16_t store_f32(float f) {
     if constexpr (DT == MI_DTYPE_BF16) {
@@ -73,7 +80,7 @@ naive_gemm_kernel(int M, int N, int K, const uint16_t* __restrict__ A,
         for (int j = 0; j < 4; ++j) {
             const int m = m0 + ty * 4 + i, n = n0 + tx * 4 + j;
             if (m < M && n < N)
-                C[(size_t)m * N + n] = store_f32<DT>(__fadd_rn(__fmul_rn(acc[i][j], alpha), beta));
+                C[(size_t)m * N + n] = store_f32<DT>(mul_add_unfused(acc[i][j], alpha, beta));
         }
 }
 

@@ -491,3 +491,44 @@ def test_tiled_split_k_random_shapes_and_alignments(mi, orc):
         C, ref, guard = _run_offset(mi, orc, config, M, N, K, offA, offB, offC)
         assert (C == ref).all(), f"{int((C != ref).sum())} elements differ"
         assert (guard == 0xEEEE).all(), "bytes outside C were written"
+
+
+# (alpha, beta, acc) for which bf16(fl(fl(acc*alpha) + beta)) != bf16(fma(acc, alpha, beta)): found by
+# search; acc = a*b with small integers, so the accumulator is exact in every kernel
+UNFUSED_CASES = [(2.1086061000823975, 6.344648361206055, 936), (3.681880235671997, -1.8010832071304321, -276),
+                 (1.982526421546936, -5.732435703277588, 187), (1.0196295976638794, -5.7203168869018555, 6),
+                 (0.6559985280036926, 5.435117244720459, -3240), (1.5280640125274658, -5.5986127853393555, 2480),
+                 (0.19303591549396515, 2.4593822956085205, -35)]
+
+
+def _bf16_bits(x):
+    u = np.asarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+@pytest.mark.parametrize("alpha,beta,acc", UNFUSED_CASES)
+def test_alpha_beta_are_two_roundings_not_an_fma(mi, orc, alpha, beta, acc):
+    """reference.h:40 computes acc * alpha + beta as a product rounded to fp32 and then a sum
+    rounded to fp32.  These inputs give a different bf16 result when the two are fused into one
+    fma, in every kernel family: tiled aligned / predicated, split-K pieces, both decode kernels,
+    the GPU golden."""
+    a = next(d for d in range(1, 65) if acc % d == 0 and abs(acc // d) <= 64)
+    b = acc // a
+    un = (np.float32(np.float32(acc) * np.float32(alpha)) + np.float32(beta)).astype(np.float32)
+    fu = np.float32(np.float64(acc) * np.float64(np.float32(alpha)) + np.float64(np.float32(beta)))
+    assert _bf16_bits(un) != _bf16_bits(fu), "the case no longer tells one fma from two roundings"
+    for M, N, K in [(64, 64, 1), (256, 256, 128), (300, 260, 200), (512, 512, 4096), (16, 256, 128), (64, 256, 256),
+                    (128, 512, 2048)]:
+        A = np.zeros((M, K), np.float32)
+        B = np.zeros((N, K), np.float32)
+        A[:, K // 2] = a
+        B[:, K // 2] = b
+        A, B = orc.from_f32(A, 0), orc.from_f32(B, 0)
+        ref = orc.reference_cpu_gemm(A, B, alpha=alpha, beta=beta)
+        assert (ref == _bf16_bits(un)).all()
+        d = Dev(mi, A, B, M, N)
+        assert (d.run_epilogue(K, alpha, beta) == ref).all(), (M, N, K)
+        p = mi.GemmParams(M, N, K, d.dA, d.dB, d.dC, alpha, beta)
+        mi.reference_gpu_gemm(p)
+        mi.synchronize()
+        assert (d.dC.to_numpy((M, N), np.uint16) == ref).all(), ("golden", M, N, K)
