@@ -213,6 +213,7 @@ CONFIGS = [
     _k(32, NS=4),
     _k(64, NS=6),
     _k(128, NS=5),
+    _m(256, 256, 2, 2, GROUP=8, DRAIN=1),
     _m(192, 192, 2, 2, DRAIN=1, EFF=0.80, EFF_E=0.91),
     _m(192, 128, 2, 2, DRAIN=1, EFF=0.74, EFF_E=0.85),
 ]
@@ -220,10 +221,11 @@ CONFIGS = [
 assert all(is_valid_config(c) for c in CONFIGS), [config_name(c) for c in CONFIGS if not is_valid_config(c)]
 assert len({config_name(c) for c in CONFIGS}) == len(CONFIGS)
 
-# Exact shapes with a tuned choice (config name), consulted before the cost model.  Empty at
-# present: the four-wave 16x16x32-MFMA kernel is ahead at every aligned shape measured
-# (8192^3, both MLP shapes, 4096^3, K = 12288 .. 28672).
-TUNED_SHAPES = {}
+# Exact shapes with a tuned choice (config name), consulted before the model.  From sweeps of
+# the 256x256 family (GROUP 4 / 8 x DRAIN 0 / 1 / 3) at the benchmark shapes: at 8192^3 and
+# N = 28672 the default is level with or ahead of the others; at K = 28672 groups 8 tiles tall
+# with the earlier drain slot are 1.7 % faster (2.426 against 2.468 ms).
+TUNED_SHAPES = {(8192, 8192, 28672): "m256x256_w2x2_g8_b1"}
 assert all(n in {config_name(c) for c in CONFIGS} for n in TUNED_SHAPES.values())
 
 # Automatic choice for decode shapes (the kernels' preconditions permitting): (largest M,
