@@ -37,11 +37,11 @@ def _write_if_changed(path: Path, text: str) -> None:
         path.write_text(text)
 
 
-def _decode_ladder(named) -> list[tuple[int, int, int, int]]:
-    """(max M, config index, max N per CU or 0, min K) steps of the automatic choice for decode shapes."""
+def _decode_ladder(named) -> list[tuple[int, int, str]]:
+    """(max M, config index, condition on N and K) steps of the automatic choice for decode shapes."""
     names = [c["name"] for c in named]
     ladder = getattr(kc, "DECODE_LADDER", [])
-    return [(m, names.index(n), lim, kmin) for m, n, lim, kmin in ladder if n in names]
+    return [(m, names.index(n), cond) for m, n, cond in ladder if n in names]
 
 
 def render_sources(configs=None) -> list[Path]:

@@ -229,11 +229,19 @@ TUNED_SHAPES = {(8192, 8192, 28672): "m256x256_w2x2_g8_b1"}
 assert all(n in {config_name(c) for c in CONFIGS} for n in TUNED_SHAPES.values())
 
 # Automatic choice for decode shapes (the kernels' preconditions permitting): (largest M,
-# config name, largest N per compute unit or 0 for any, smallest K), first match wins.
-# Up to M = 32 the single-pass kernel; above, the split-K kernel measured ahead of it
-# (M = 64: 30 us against 33 us).  Above M = 128 the tiled kernels with split-K take over
-# (256 x 8192 x 8192: 48.8 us as 256x128 tiles x 4 pieces; a 256-row variant of the decode
-# kernel, one slab in flight per CU, took 61 us and was dropped).
-DECODE_LADDER = [(16, "s16x32_n5", 0, 0), (32, "s32x32_n4", 0, 0), (64, "k64x128_n6", 0, 0),
-                 (128, "k128x128_n5", 0, 0)]
-assert all(n in {config_name(c) for c in CONFIGS} for _, n, _, _ in DECODE_LADDER)
+# config name, further condition on N and K as a C expression), first match wins; shapes that
+# match no step go to the tiled kernels (with split-K where the time model wants it).
+# Up to M = 32 the single-pass kernel, always (16 x 1024 x 8192: 10.6 us against 13.1 us tiled;
+# 16 x 8192 x 28672: 80 against 87).  The split-K decode kernels are ahead for wide B
+# (N = 28672: 83 against 120 us at M = 64, 113 against 122 us at M = 128) and level at
+# N = 8192 for 8192 <= K <= 16384; the tiled kernels win for narrow B (M = 128, N <= 4096:
+# 11-20 against 14-21 us; M = 64, N = 2048: 12.5 against 14.2 us) and for very long K
+# (8192 x 28672: 97 against 105 us at M = 64, 106 against 136 us at M = 128).
+DECODE_LADDER = [(16, "s16x32_n5", "true"), (32, "s32x32_n4", "true"),
+                 (64, "k64x128_n6", "N >= 4096 && K < 24576"),
+                 (128, "k128x128_n5", "N >= 16384 || (N >= 8192 && K >= 8192 && K < 24576)"),
+                 # very long K: 128x256 tiles (one row of tiles covers M, B is read once) in split-K
+                 # pieces: 97 / 106 us at M = 64 / 128 against 105 / 136 us for the decode kernels
+                 # and 115-143 us for the other tiles, between which the time model cannot tell
+                 (128, "m128x256_w2x2_g4_b1", "N >= 4096 && K >= 24576")]
+assert all(n in {config_name(c) for c in CONFIGS} for _, n, _ in DECODE_LADDER)
