@@ -532,3 +532,24 @@ def test_alpha_beta_are_two_roundings_not_an_fma(mi, orc, alpha, beta, acc):
         mi.reference_gpu_gemm(p)
         mi.synchronize()
         assert (d.dC.to_numpy((M, N), np.uint16) == ref).all(), ("golden", M, N, K)
+
+
+def test_automatic_choice_across_regimes_bit_exact(mi, orc):
+    """The shape -> kernel choice has many branches (decode ladder with its N / K conditions,
+    tuned shapes, tile model, split-K pieces, aligned / predicated twins).  Shapes on both sides
+    of each boundary, integer fill, automatic choice: every result must match the oracle's bits,
+    whichever kernel ran."""
+    shapes = []
+    for M in (1, 16, 17, 32, 33, 64, 65, 128, 129, 256, 257):
+        shapes += [(M, 4096, 4096), (M, 1024, 8192), (M, 8192, 512), (M, 4100, 1088)]
+    shapes += [(64, 4096, 24576), (128, 4096, 24576), (96, 16384, 1024), (128, 8192, 8192), (48, 8192, 2048),
+               (130, 4096, 24640), (512, 512, 4096), (3000, 3000, 264), (384, 384, 6016), (192, 8192, 2048)]
+    seen = set()
+    for M, N, K in shapes:
+        cfg = mi.select_config(M, N, K)
+        seen.add(mi.config_name(cfg))
+        print(f"case M={M} N={N} K={K} -> {mi.config_name(cfg)} grid {mi.config_grid(cfg, M, N, K)}", flush=True)
+        check(mi, orc, M, N, K, "int", exact=True)
+    # the sweep is only worth its time if it reaches the different kernel families
+    assert {"s16x32_n5", "s32x32_n4", "k64x128_n6", "k128x128_n5"} <= seen, seen
+    assert any(n.startswith("m128x256") for n in seen) and any(n.startswith("m128x128") for n in seen), seen
