@@ -164,15 +164,41 @@ int check_args(int config, int dtype, int M, int N, int K, const void* A, const 
     return MI_OK;
 }
 
+// The automatic choice is a pure function of the shape and three flags and costs 1-3 us of
+// host time (the time model runs over every candidate and piece count), which shows when
+// small GEMMs are launched back to back: the last few answers are kept per thread, keyed on
+// all of its inputs.  (No pointer or other per-call state is cached.)
+struct Choice {
+    int M, N, K, flags, requested;   // key; requested = the caller's config (MI_CONFIG_AUTO or an index)
+    int config, splits, k_per_split;
+};
+Choice choose(int requested, int M, int N, int K, bool streamable, bool splittable, bool ptr_aligned) {
+    static thread_local Choice memo[4] = {};
+    static thread_local int next = 0;
+    const int flags = (streamable ? 1 : 0) | (splittable ? 2 : 0) | (ptr_aligned ? 4 : 0);
+    for (const Choice& c : memo)
+        if (c.M == M && c.N == N && c.K == K && c.flags == flags && c.requested == requested && c.splits > 0)
+            return c;
+    Choice c{M, N, K, flags, requested, requested, 1, K};
+    if (requested == MI_CONFIG_AUTO)
+        c.config = mi::select_kernel(M, N, K, streamable, splittable, ptr_aligned, compute_units());
+    const mi::KernelEntry& e = mi::kKernels[c.config];
+    if (e.kind == mi::KIND_MFMA16)
+        c.splits = choose_tile_splits(e, M, N, K, splittable, ptr_aligned, compute_units(), &c.k_per_split);
+    memo[next] = c;
+    next = (next + 1) & 3;
+    return c;
+}
+
 // One GEMM launch (two for split-K): argument checks, kernel choice, aligned / predicated twin.
 int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const void* B, void* C,
              int* DB, float alpha, float beta, void* stream) {
     int rc = check_args(config, dtype, M, N, K, A, B, C);
     if (rc != MI_OK) return rc;
     const bool streamable = shape_is_streamable(M, N, K, A, B, C);
-    if (config == MI_CONFIG_AUTO)
-        config = mi::select_kernel(M, N, K, streamable, shape_is_splittable(N, C, DB),
-                                   aligned16(A) && aligned16(B) && aligned16(C), compute_units());
+    const Choice choice = choose(config, M, N, K, streamable, shape_is_splittable(N, C, DB),
+                                 aligned16(A) && aligned16(B) && aligned16(C));
+    config = choice.config;
     const mi::KernelEntry& e = mi::kKernels[config];
 
     mi::GemmArgs args;
@@ -229,8 +255,8 @@ int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const vo
     if (!fn) return fail(MI_ERR_UNSUPPORTED, "config %s has no %s kernel for dtype %d", e.name,
                          edge ? "predicated" : "aligned", dtype);
     if (e.kind == mi::KIND_MFMA16) {
-        args.splits = choose_tile_splits(e, M, N, K, shape_is_splittable(N, C, DB),
-                                         aligned16(A) && aligned16(B) && aligned16(C), compute_units(), &args.k_per_split);
+        args.splits = choice.splits;
+        args.k_per_split = choice.k_per_split;
         if (args.splits > 1) {
             hipError_t we = ensure_workspace((size_t)args.splits * M * N * sizeof(float), &args.ws);
             if (we != hipSuccess)
