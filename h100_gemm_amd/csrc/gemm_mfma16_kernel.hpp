@@ -457,8 +457,13 @@ gemm_mfma16_kernel(const GemmArgs p) {
         };
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");   // all waves done with the last stage
         unsigned char* stg = lds + wave * (TM * TN * 2);
+        // In pieces of 32 rows (where the row layout allows): the stores of one piece drain
+        // while the next is converted, instead of 128 KB per CU queueing up at once.
+        constexpr int CH_ROWS = (POW2 && TM % 32 == 0 && 32 % (64 / CPR) == 0) ? 32 : TM;
 #pragma unroll
-        for (int i = 0; i < MI; ++i) {
+        for (int c = 0; c < TM / CH_ROWS; ++c) {
+#pragma unroll
+        for (int i = c * (CH_ROWS / 16); i < (c + 1) * (CH_ROWS / 16); ++i) {
             const int row = i * 16 + l16;
 #pragma unroll
             for (int j = 0; j < NI; ++j) {
@@ -471,7 +476,7 @@ gemm_mfma16_kernel(const GemmArgs p) {
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
-        for (int r = 0; r < TM * CPR / 64; ++r) {
+        for (int r = c * (CH_ROWS * CPR / 64); r < (c + 1) * (CH_ROWS * CPR / 64); ++r) {
             // chunk r*64 + lane of the wave tile, rows first
             const int idx = r * 64 + lane;
             const int row = POW2 ? r * (64 / CPR) + lane / CPR : idx / CPR;
@@ -495,6 +500,7 @@ gemm_mfma16_kernel(const GemmArgs p) {
                     }
                 }
             }
+        }
         }
     };
     if constexpr (SPLITK) {
