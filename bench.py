@@ -83,6 +83,35 @@ def cpu_baseline(orc, A, B, budget_tiles: int) -> dict:
                       f"{dt * total_tiles / len(tiles):.0f} s"}
 
 
+def sclk_under_load(launch_batch, sync) -> float | None:
+    """Shader clock in MHz as the driver's management interface reports it while the GPU runs
+    this workload (the chip is power limited: the sustained clock, not the peak clock, is what
+    the measured rate is made of).  None when the tool is missing or prints something else."""
+    import re
+    import shutil
+    import subprocess
+    smi = shutil.which("rocm-smi") or "/opt/rocm/bin/rocm-smi"
+    if not os.path.exists(smi):
+        return None
+    # not under a profiler: the child process would inherit its tool library
+    if any(k.startswith(("ROCPROF", "ROCP_", "ROCTRACER")) for k in os.environ):
+        return None
+    try:
+        proc = subprocess.Popen([smi, "--showclocks", "--json"], stdout=subprocess.PIPE,
+                                stderr=subprocess.DEVNULL, text=True)
+        t_end = time.perf_counter() + 20.0
+        while proc.poll() is None and time.perf_counter() < t_end:
+            launch_batch()
+            sync()
+        if proc.poll() is None:
+            proc.kill()
+        out = proc.communicate()[0]
+        m = re.search(r'"sclk clock speed:"\s*:\s*"\((\d+(?:\.\d+)?)Mhz\)"', out)
+        return float(m.group(1)) if m else None
+    except (OSError, ValueError):
+        return None
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -99,6 +128,8 @@ def main() -> int:
     ap.add_argument("--config", default=None, help="kernel configuration name or index (default: library's choice)")
     ap.add_argument("--cpu-tiles", type=int, default=2048, help="64x64 tiles in the CPU baseline sample (0 = skip)")
     ap.add_argument("--check-tiles", type=int, default=64, help="64x64 tiles verified against the oracle (0 = skip)")
+    ap.add_argument("--no-sclk", dest="sclk", action="store_false",
+                    help="do not sample the shader clock under load after the timed region")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain device-to-device copy of 256 MiB (a kernel of known HBM "
                          "traffic, for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
@@ -164,6 +195,11 @@ def main() -> int:
     ms_total = timer.report_last_ms()
     ms_per_step = ms_total / a.steps
 
+    def launch_batch():      # ~30 ms of the same launches, outside the timed region
+        for i in range(max(1, int(30.0 / ms_per_step))):
+            mi.gpu_gemm(params[i % len(params)], config=cfg)
+    sclk = sclk_under_load(launch_batch, mi.synchronize) if a.sclk else None
+
     # correctness of what was just timed, on a sample of tiles
     violations = None
     if a.check_tiles > 0:
@@ -196,7 +232,8 @@ def main() -> int:
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic" + (", 3 rotating copies of B" if hbm_bound else ""),
         "config": {"workload": f"{a.workload}: M={M} N={N} K={K}, A,B {fill} seeded bf16, fp32 accumulate, bf16 out",
                    "kernel_config": mi.config_name(cfg), "device": props["name"] or props["arch"],
-                   "compute_units": props["compute_units"], "peak_clock_mhz": props["clock_khz"] / 1000},
+                   "compute_units": props["compute_units"], "peak_clock_mhz": props["clock_khz"] / 1000,
+                   "sclk_mhz_under_load": sclk},
         "pct_of_bf16_mfma_peak": 100.0 * tflops / PEAK_BF16_TFLOPS,
         "achieved_gbs_algorithmic": gbs,
         "tolerance_violations": violations,
