@@ -143,7 +143,9 @@ def main() -> int:
         print("bench.py: launched with WORLD_SIZE > 1; one GPU only", file=sys.stderr)
         return 2
 
-    import h100_gemm_amd as mi          # raises if libmi_gemm.so is not built
+    import __graft_entry__
+    __graft_entry__.ensure_built()      # uses what is built; compiles only if nothing is
+    import h100_gemm_amd as mi          # raises if libmi_gemm.so is missing
     from oracle import oracle as orc    # checker + CPU baseline only
 
     M, N, K, fill = WORKLOADS[a.workload]

@@ -37,6 +37,8 @@ def orc():
 
 @pytest.fixture(scope="session")
 def mi():
+    import __graft_entry__
+    __graft_entry__.ensure_built()      # uses what is built; compiles only if nothing is
     import h100_gemm_amd
     h100_gemm_amd._lib.load()
     return h100_gemm_amd
