@@ -100,42 +100,55 @@ int choose_tile_splits(const mi::KernelEntry& e, int M, int N, int K, bool split
     return mi::best_splits(e, M, N, K, true, ptr_aligned, cus, k_per_split, nullptr);
 }
 
-// fp32 partial-sum workspace of the split-K kernels: one buffer per process, grown on
+// fp32 partial-sum workspace of the split-K kernels: one buffer per device, grown on
 // demand.  Launches that use it are ordered on their stream; callers that run split-K
-// launches on several streams at once must serialise them.
+// launches on several streams of one device at once must serialise them.  Workspace and
+// CU count belong to the device that is current when the call is made.
+constexpr int kMaxDevices = 64;
+struct DeviceState {
+    float* ws = nullptr;
+    size_t ws_bytes = 0;
+    int cus = 0;
+};
 std::mutex g_ws_mutex;
-float* g_ws = nullptr;
-size_t g_ws_bytes = 0;
-int g_cus = 0;
+DeviceState g_dev[kMaxDevices];
+
+DeviceState& device_state() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) dev = 0;
+    return g_dev[dev];
+}
 
 hipError_t ensure_workspace(size_t bytes, float** out) {
     std::lock_guard<std::mutex> lock(g_ws_mutex);
-    if (bytes > g_ws_bytes) {
-        if (g_ws) {
-            hipError_t e = hipFree(g_ws);      // waits for work that may still use it
-            g_ws = nullptr;
-            g_ws_bytes = 0;
+    DeviceState& st = device_state();
+    if (bytes > st.ws_bytes) {
+        if (st.ws) {
+            hipError_t e = hipFree(st.ws);     // waits for work that may still use it
+            st.ws = nullptr;
+            st.ws_bytes = 0;
             if (e != hipSuccess) return e;
         }
         const size_t want = bytes < (size_t)(32u << 20) ? (size_t)(32u << 20) : bytes;
-        hipError_t e = hipMalloc((void**)&g_ws, want);
+        hipError_t e = hipMalloc((void**)&st.ws, want);
         if (e != hipSuccess) return e;
-        g_ws_bytes = want;
+        st.ws_bytes = want;
     }
-    *out = g_ws;
+    *out = st.ws;
     return hipSuccess;
 }
 
 int compute_units() {
-    if (g_cus == 0) {
+    DeviceState& st = device_state();
+    if (st.cus == 0) {
         int dev = 0, n = 0;
         if (hipGetDevice(&dev) == hipSuccess &&
             hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-            g_cus = n;
+            st.cus = n;
         else
-            g_cus = 256;
+            st.cus = 256;
     }
-    return g_cus;
+    return st.cus;
 }
 
 // The aligned kernels assume full tiles, K a multiple of two K steps, 16-byte aligned
@@ -169,22 +182,24 @@ int check_args(int config, int dtype, int M, int N, int K, const void* A, const 
 // small GEMMs are launched back to back: the last few answers are kept per thread, keyed on
 // all of its inputs.  (No pointer or other per-call state is cached.)
 struct Choice {
-    int M, N, K, flags, requested;   // key; requested = the caller's config (MI_CONFIG_AUTO or an index)
+    int M, N, K, flags, requested, cus;   // key; requested = the caller's config (MI_CONFIG_AUTO or an index)
     int config, splits, k_per_split;
 };
 Choice choose(int requested, int M, int N, int K, bool streamable, bool splittable, bool ptr_aligned) {
     static thread_local Choice memo[4] = {};
     static thread_local int next = 0;
     const int flags = (streamable ? 1 : 0) | (splittable ? 2 : 0) | (ptr_aligned ? 4 : 0);
+    const int cus = compute_units();
     for (const Choice& c : memo)
-        if (c.M == M && c.N == N && c.K == K && c.flags == flags && c.requested == requested && c.splits > 0)
+        if (c.M == M && c.N == N && c.K == K && c.flags == flags && c.requested == requested && c.cus == cus &&
+            c.splits > 0)
             return c;
-    Choice c{M, N, K, flags, requested, requested, 1, K};
+    Choice c{M, N, K, flags, requested, cus, requested, 1, K};
     if (requested == MI_CONFIG_AUTO)
-        c.config = mi::select_kernel(M, N, K, streamable, splittable, ptr_aligned, compute_units());
+        c.config = mi::select_kernel(M, N, K, streamable, splittable, ptr_aligned, cus);
     const mi::KernelEntry& e = mi::kKernels[c.config];
     if (e.kind == mi::KIND_MFMA16)
-        c.splits = choose_tile_splits(e, M, N, K, splittable, ptr_aligned, compute_units(), &c.k_per_split);
+        c.splits = choose_tile_splits(e, M, N, K, splittable, ptr_aligned, cus, &c.k_per_split);
     memo[next] = c;
     next = (next + 1) & 3;
     return c;
