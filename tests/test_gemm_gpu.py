@@ -347,6 +347,21 @@ def test_harness_programs(mi):
     assert re.search(r"Average elapsed time: \(\s*[\d.]+\) s, performance: \(\s*[\d.]+\) TFLOPS\. size: \(1024\)\.", r.stdout)
 
 
+def test_mfma_ceiling_program(mi):
+    """The MFMA-only yardstick program: same issue rate for every data set (a 16x16x32 MFMA is
+    16 cycles), and zeros must not be slower than random operands (the chip is power limited)."""
+    exe = ROOT / "h100_gemm_amd" / "harness" / "mfma_ceiling"
+    assert exe.exists(), f"{exe} is not built (make -C h100_gemm_amd/harness)"
+    out = subprocess.run([str(exe), "60"], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stdout + out.stderr
+    rows = re.findall(r"^(.+?)\s+([\d.]+) cycles per MFMA, clock ([\d.]+) GHz, (\d+) TFLOP/s$", out.stdout, re.M)
+    assert [r[0].strip() for r in rows] == ["zeros", "uniform [-1,1) bf16", "normal(0,1) bf16"], out.stdout
+    for name, cyc, clock, tf in rows:
+        assert 16.0 <= float(cyc) <= 17.5, (name, cyc)
+        assert 0.5 <= float(clock) <= 2.6, (name, clock)
+    assert int(rows[0][3]) >= int(rows[1][3]) * 0.98, rows
+
+
 def test_vendor_side_by_side_program(mi):
     """kernel 0 (vendor BLAS, linked into this program only) and kernel 1 on the same buffers:
     the loop of matmul_h100_optimal.cu:157-217 with the comparison of :177-180 switched on."""
