@@ -160,6 +160,16 @@ def test_ragged_and_tiny_shapes(mi, orc, M, N, K):
     check(mi, orc, M, N, K, "uniform")
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 1, 4194303), (3, 130, 1048577), (1 << 22, 8, 8), (8, 1 << 22, 8),
+                                   (1, 1 << 23, 16), (1 << 21, 1, 64), (20000, 20000, 1), (600000, 8, 2048), (8, 600000, 2048)])
+def test_extreme_aspect_ratios(mi, orc, M, N, K):
+    # the largest K the library accepts (K * 512 < 2^31), millions of tile rows / columns
+    # (64-bit row offsets, 32-bit offsets inside a tile's panel), a single column, K = 1,
+    # operands of 2.4 GB (byte offsets past 2^31)
+    fill = "uniform" if K > 100000 else "int"
+    check(mi, orc, M, N, K, fill, exact=fill == "int")
+
+
 def test_k_tail_with_page_aligned_matrix_end(mi, orc):
     # odd K with M a multiple of 2048: the last element of A sits right below a 4 KiB
     # boundary of the allocation; the kernel must fetch it without reading past the matrix

@@ -87,7 +87,14 @@ def test_argument_validation_needs_no_device(mi):
     assert L.mi_gemm_bf16(8, 8, 8, None, 1, 1, None, None) == mi._lib.MI_ERR_INVALID
     assert L.mi_gemm_ex(999, bf, 8, 8, 8, 1, 1, 1, None, None) == mi._lib.MI_ERR_INVALID
     assert L.mi_gemm_ex(-1, 7, 8, 8, 8, 1, 1, 1, None, None) == mi._lib.MI_ERR_INVALID
+    # size limits: each matrix below 2^31 elements (int indices, as reference.h:30,40), and a
+    # 256-row panel of K-long rows within the 32-bit byte offsets of one buffer descriptor
     assert L.mi_gemm_ex(-1, bf, 70000, 70000, 8, 1, 1, 1, None, None) == mi._lib.MI_ERR_INVALID
+    assert b"2^31" in L.mi_last_error()
+    assert L.mi_gemm_ex(-1, bf, 65536, 8, 32768, 1, 1, 1, None, None) == mi._lib.MI_ERR_INVALID      # M*K = 2^31
+    assert L.mi_gemm_ex(-1, bf, 8, 65536, 32768, 1, 1, 1, None, None) == mi._lib.MI_ERR_INVALID      # N*K = 2^31
+    assert L.mi_gemm_ex(-1, bf, 1, 1, 4194304, 1, 1, 1, None, None) == mi._lib.MI_ERR_INVALID        # K*512 = 2^31
+    assert b"K too large" in L.mi_last_error()
     assert L.mi_reference_gpu_gemm(bf, 8, -1, 8, 1, 1, 1, 1.0, 0.0, None) == mi._lib.MI_ERR_INVALID
     assert L.mi_gemm_epilogue(-1, bf, 8, 8, 8, 1, 1, 1, 1.0, 0.0, 2, None) == mi._lib.MI_ERR_INVALID
     assert b"layout" in L.mi_last_error()
