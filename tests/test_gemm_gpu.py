@@ -242,6 +242,47 @@ def test_random_shapes_and_alignments_every_tiled_kind(mi, orc):
         assert (guard == 0xEEEE).all(), "bytes outside C were written"
 
 
+def test_non_default_streams_and_host_threads(mi, orc):
+    """The ABI's stream argument: two host threads, each launching on a stream of its own
+    (created with default priority) and waiting with mi_stream_sync; shapes that use no
+    shared workspace (concurrent split-K launches are documented as the caller's to order)."""
+    import ctypes
+    import threading
+    hip = ctypes.CDLL("libamdhip64.so")
+    L = mi._lib.load()
+    shapes = [(512, 512, 512), (1024, 768, 256), (16, 2048, 1024), (257, 515, 77), (768, 1280, 384)]
+    errors = []
+
+    def worker(seed):
+        try:
+            stream = ctypes.c_void_p()
+            assert hip.hipStreamCreate(ctypes.byref(stream)) == 0
+            for rep in range(6):
+                M, N, K = shapes[(rep + seed) % len(shapes)]
+                A, B = make_inputs(orc, M, N, K, "int", seed=69 + seed)
+                ref = orc.reference_cpu_gemm(A, B)
+                dA, dB = mi.DeviceBuffer.from_numpy(A), mi.DeviceBuffer.from_numpy(B)
+                dC = mi.DeviceBuffer(M * N * 2)
+                dC.fill_bytes(0xFF)
+                mi._lib.check(L.mi_gemm_ex(-1, 0, M, N, K, dA.ptr, dB.ptr, dC.ptr, None, stream))
+                mi._lib.check(L.mi_stream_sync(stream))
+                C = dC.to_numpy((M, N), np.uint16)
+                if not (C == ref).all():
+                    errors.append(f"thread {seed} rep {rep} {M}x{N}x{K}: {int((C != ref).sum())} elements differ")
+                for b in (dA, dB, dC):
+                    b.free()
+            assert hip.hipStreamDestroy(stream) == 0
+        except Exception as e:      # surfaced in the main thread
+            errors.append(f"thread {seed}: {type(e).__name__}: {e}")
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+
+
 def test_output_buffer_is_not_overrun(mi, orc):
     M, N, K = 257, 515, 77
     A, B = make_inputs(orc, M, N, K, "int")
