@@ -283,6 +283,42 @@ def test_non_default_streams_and_host_threads(mi, orc):
     assert not errors, errors
 
 
+def test_hip_graph_replay_of_gemm_launches(mi, orc):
+    """Launches that need no workspace allocate nothing and can be captured into a HIP graph:
+    a tiled and a decode GEMM recorded on a capturing stream, replayed three times with eager
+    work and synchronisation in between, every replay compared with the eager result."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    L = mi._lib.load()
+    cases = [(512, 512, 512), (16, 2048, 1024), (300, 200, 100)]
+    bufs, want = [], []
+    for M, N, K in cases:
+        A, B = make_inputs(orc, M, N, K, "int")
+        d = Dev(mi, A, B, M, N)
+        want.append(d.run(K).copy())                       # eager result (also loads the kernels)
+        assert (want[-1] == orc.reference_cpu_gemm(A, B)).all()
+        bufs.append((d, M, N, K))
+    stream, graph, gexec = ctypes.c_void_p(), ctypes.c_void_p(), ctypes.c_void_p()
+    assert hip.hipStreamCreate(ctypes.byref(stream)) == 0
+    assert hip.hipStreamBeginCapture(stream, 0) == 0       # hipStreamCaptureModeGlobal
+    rcs = [L.mi_gemm_ex(-1, 0, M, N, K, d.dA.ptr, d.dB.ptr, d.dC.ptr, None, stream) for d, M, N, K in bufs]
+    assert hip.hipStreamEndCapture(stream, ctypes.byref(graph)) == 0
+    assert rcs == [0] * len(cases), rcs
+    assert hip.hipGraphInstantiate(ctypes.byref(gexec), graph, None, None, ctypes.c_size_t(0)) == 0
+    for replay in range(3):
+        for d, M, N, K in bufs:
+            d.dC.fill_bytes(0xFF)                          # eager work between the replays
+        mi.synchronize()
+        assert hip.hipGraphLaunch(gexec, stream) == 0
+        mi._lib.check(L.mi_stream_sync(stream))
+        for (d, M, N, K), ref in zip(bufs, want):
+            C = d.dC.to_numpy((M, N), np.uint16)
+            assert (C == ref).all(), f"replay {replay} {M}x{N}x{K}: {int((C != ref).sum())} elements differ"
+    assert hip.hipGraphExecDestroy(gexec) == 0
+    assert hip.hipGraphDestroy(graph) == 0
+    assert hip.hipStreamDestroy(stream) == 0
+
+
 def test_output_buffer_is_not_overrun(mi, orc):
     M, N, K = 257, 515, 77
     A, B = make_inputs(orc, M, N, K, "int")
