@@ -319,6 +319,46 @@ def test_hip_graph_replay_of_gemm_launches(mi, orc):
     assert hip.hipStreamDestroy(stream) == 0
 
 
+SPECIAL_SHAPES = [(256, 256, 128), (130, 70, 72), (16, 2048, 1024), (64, 4096, 8192), (256, 256, 4096)]
+
+
+@pytest.mark.parametrize("M,N,K", SPECIAL_SHAPES)
+def test_overflow_underflow_and_nan_follow_ieee(mi, orc, M, N, K):
+    """Every epilogue (direct, predicated, in-LDS reduction, split-K reduction) rounds like the
+    oracle at the ends of the range: fp16 overflow to +-inf, fp32 accumulator overflow to inf
+    in bf16, fp16 results in the subnormal range (round to nearest even there too), and a NaN
+    in one row of A makes exactly that row of C NaN."""
+    FP16, BF16 = orc.FP16, orc.BF16
+    # fp16: +-(64 * 64 * K) is far above 65504
+    A = orc.fill_constant((M, K), 64.0, FP16)
+    B = orc.fill_constant((N, K), 64.0, FP16)
+    B[1::2] = orc.fill_constant((N, K), -64.0, FP16)[1::2]
+    C = Dev(mi, A, B, M, N).run(K, dtype=FP16)
+    ref = orc.reference_cpu_gemm(A, B, dtype=FP16)
+    assert set(np.unique(ref)) <= {0x7C00, 0xFC00} and (C == ref).all()
+    # bf16: 1e19 * 1e19 * K overflows the fp32 accumulator
+    A = orc.fill_constant((M, K), 1e19, BF16)
+    B = orc.fill_constant((N, K), 1e19, BF16)
+    C = Dev(mi, A, B, M, N).run(K)
+    ref = orc.reference_cpu_gemm(A, B)
+    assert (ref == 0x7F80).all() and (C == ref).all()
+    # fp16 subnormal results: products 2^-13 * 2^-12 * {1, 0, 1, ...} sum to small multiples of 2^-25
+    A = orc.fill_constant((M, K), 2.0 ** -13, FP16)
+    B = np.zeros((N, K), np.uint16)
+    for j in range(N):
+        B[j, :(j % 7) + 1] = orc.fill_constant((1,), 2.0 ** -12, FP16)[0]     # (j % 7 + 1) * 2^-25
+    C = Dev(mi, A, B, M, N).run(K, dtype=FP16)
+    ref = orc.reference_cpu_gemm(A, B, dtype=FP16)
+    assert len(np.unique(ref)) >= 4 and (ref < 0x0400).all()                    # subnormal halves, several values
+    assert (C == ref).all(), f"{int((C != ref).sum())} elements differ"
+    # NaN in row 3 of A (if there is one)
+    A, B = make_inputs(orc, M, N, K, "int")
+    row = min(3, M - 1)
+    A[row, K // 2] = 0x7FC0
+    C = orc.to_f32(Dev(mi, A, B, M, N).run(K))
+    assert np.isnan(C[row]).all() and not np.isnan(np.delete(C, row, axis=0)).any()
+
+
 def test_output_buffer_is_not_overrun(mi, orc):
     M, N, K = 257, 515, 77
     A, B = make_inputs(orc, M, N, K, "int")
