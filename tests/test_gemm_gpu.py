@@ -326,8 +326,9 @@ SPECIAL_SHAPES = [(256, 256, 128), (130, 70, 72), (16, 2048, 1024), (64, 4096, 8
 def test_overflow_underflow_and_nan_follow_ieee(mi, orc, M, N, K):
     """Every epilogue (direct, predicated, in-LDS reduction, split-K reduction) rounds like the
     oracle at the ends of the range: fp16 overflow to +-inf, fp32 accumulator overflow to inf
-    in bf16, fp16 results in the subnormal range (round to nearest even there too), and a NaN
-    in one row of A makes exactly that row of C NaN."""
+    in bf16, fp16 results in the subnormal range (round to nearest even there too), subnormal
+    inputs and sums kept (nothing is flushed to zero), and a NaN in one row of A makes exactly
+    that row of C NaN."""
     FP16, BF16 = orc.FP16, orc.BF16
     # fp16: +-(64 * 64 * K) is far above 65504
     A = orc.fill_constant((M, K), 64.0, FP16)
@@ -351,6 +352,18 @@ def test_overflow_underflow_and_nan_follow_ieee(mi, orc, M, N, K):
     ref = orc.reference_cpu_gemm(A, B, dtype=FP16)
     assert len(np.unique(ref)) >= 4 and (ref < 0x0400).all()                    # subnormal halves, several values
     assert (C == ref).all(), f"{int((C != ref).sum())} elements differ"
+    # subnormal inputs (bf16 2^-127, fp16 2^-15) are not flushed, nor are sums in the
+    # subnormal range of fp32 / of the storage type
+    for dtype, tiny, big, pa, pb in ((BF16, 0x0040, 2.0 ** 100, 2.0 ** -70, 2.0 ** -65),
+                                    (FP16, 0x0200, 2.0 ** 10, 2.0 ** -14, 2.0 ** -14)):
+        A = np.full((M, K), tiny, np.uint16)
+        B = orc.fill_constant((N, K), big, dtype)
+        ref = orc.reference_cpu_gemm(A, B, dtype=dtype)
+        assert (ref != 0).all() and (Dev(mi, A, B, M, N).run(K, dtype=dtype) == ref).all()
+        A = orc.fill_constant((M, K), pa, dtype)
+        B = orc.fill_constant((N, K), pb, dtype)
+        ref = orc.reference_cpu_gemm(A, B, dtype=dtype)
+        assert (ref != 0).all() and (Dev(mi, A, B, M, N).run(K, dtype=dtype) == ref).all()
     # NaN in row 3 of A (if there is one)
     A, B = make_inputs(orc, M, N, K, "int")
     row = min(3, M - 1)
