@@ -9,6 +9,7 @@ tile of reference.h is independent, so a sampled tile holds exactly the full run
 plus size-independent properties (row/column permutation equivariance, identity, run-to-run
 determinism).
 """
+import os
 import re
 import subprocess
 from pathlib import Path
@@ -230,7 +231,8 @@ def test_random_shapes_and_alignments_every_tiled_kind(mi, orc):
         if c["KIND"] in ("tile", "ring", "mfma16", "ring16"):
             picks.setdefault((c["KIND"], c.get("DRAIN", 0) > 0, c["BN"] == 192), i)
     configs = [-1] + sorted(picks.values())
-    for it in range(36):
+    # MI_GEMM_RANDOM_CASES=<n> turns this into a longer sweep (36 cases by default)
+    for it in range(int(os.environ.get("MI_GEMM_RANDOM_CASES", "36"))):
         M = int(rng.integers(1, 700))
         N = int(rng.integers(1, 700))
         K = int(rng.choice([rng.integers(1, 64), rng.integers(64, 400), 128 * rng.integers(1, 5) + rng.integers(0, 9)]))
