@@ -14,6 +14,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
+#include <vector>
 
 #include "../../include/mi_gemm.h"
 #include "gemm_kernel.hpp"
@@ -177,6 +178,48 @@ int check_args(int config, int dtype, int M, int N, int K, const void* A, const 
     return MI_OK;
 }
 
+// Tuned shapes from a file: MI_GEMM_TUNED_FILE names a text file with one `M N K config-name`
+// per line (# starts a comment), read once, on first use.  A shape listed there skips the
+// time model when its configuration can run the call (the decode kernels have preconditions);
+// lines that do not parse or name no compiled configuration are ignored.  Keyed on all of
+// M, N and K (the reference keys its cached descriptors on M alone, matmul_utils.cuh:49-51).
+struct TunedEntry {
+    int M, N, K, config;
+};
+const std::vector<TunedEntry>& tuned_entries() {
+    static const std::vector<TunedEntry> table = [] {
+        std::vector<TunedEntry> t;
+        const char* path = getenv("MI_GEMM_TUNED_FILE");
+        FILE* f = path && *path ? fopen(path, "r") : nullptr;
+        if (!f) return t;
+        char line[256];
+        while (fgets(line, sizeof(line), f)) {
+            if (char* hash = strchr(line, '#')) *hash = 0;
+            int M = 0, N = 0, K = 0;
+            char name[128];
+            if (sscanf(line, "%d %d %d %127s", &M, &N, &K, name) != 4 || M <= 0 || N <= 0 || K <= 0) continue;
+            for (int i = 0; i < mi::kNumKernels; ++i)
+                if (strcmp(name, mi::kKernels[i].name) == 0) {
+                    t.push_back({M, N, K, i});
+                    break;
+                }
+        }
+        fclose(f);
+        return t;
+    }();
+    return table;
+}
+// config for (M, N, K) from the tuned file, or -1
+int tuned_config(int M, int N, int K, bool streamable) {
+    for (const TunedEntry& t : tuned_entries()) {
+        if (t.M != M || t.N != N || t.K != K) continue;
+        const mi::KernelEntry& e = mi::kKernels[t.config];
+        if ((e.kind == mi::KIND_SKINNY || e.kind == mi::KIND_STREAM) && (!streamable || M > e.BM)) continue;
+        return t.config;
+    }
+    return -1;
+}
+
 // The automatic choice is a pure function of the shape and three flags and costs 1-3 us of
 // host time (the time model runs over every candidate and piece count), which shows when
 // small GEMMs are launched back to back: the last few answers are kept per thread, keyed on
@@ -195,8 +238,10 @@ Choice choose(int requested, int M, int N, int K, bool streamable, bool splittab
             c.splits > 0)
             return c;
     Choice c{M, N, K, flags, requested, cus, requested, 1, K};
-    if (requested == MI_CONFIG_AUTO)
-        c.config = mi::select_kernel(M, N, K, streamable, splittable, ptr_aligned, cus);
+    if (requested == MI_CONFIG_AUTO) {
+        c.config = tuned_config(M, N, K, streamable);
+        if (c.config < 0) c.config = mi::select_kernel(M, N, K, streamable, splittable, ptr_aligned, cus);
+    }
     const mi::KernelEntry& e = mi::kKernels[c.config];
     if (e.kind == mi::KIND_MFMA16)
         c.splits = choose_tile_splits(e, M, N, K, splittable, ptr_aligned, cus, &c.k_per_split);
@@ -352,8 +397,13 @@ int mi_gemm_config_grid(int config, int M, int N, int K) {
 int mi_gemm_select_config(int dtype, int M, int N, int K) {
     (void)dtype;
     // pointer alignment is unknown here: assume the usual 256-byte aligned allocations
-    return mi::select_kernel(M, N, K, N % 4 == 0 && K % 64 == 0, N % 4 == 0, true, compute_units());
+    const bool streamable = N % 4 == 0 && K % 64 == 0;
+    const int tuned = tuned_config(M, N, K, streamable);
+    if (tuned >= 0) return tuned;
+    return mi::select_kernel(M, N, K, streamable, N % 4 == 0, true, compute_units());
 }
+
+int mi_gemm_tuned_entries(void) { return (int)tuned_entries().size(); }
 
 size_t mi_gemm_trace_words(int M, int N, int K) {
     // enough for whichever kernel configuration ends up running the shape

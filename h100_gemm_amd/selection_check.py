@@ -8,7 +8,8 @@ against the best candidate and every candidate's time.  A tuning aid for the con
 (``gemm_tuner.py:82-133``) for the choice between compiled kernels instead of between
 template parameters.
 
-    python -m h100_gemm_amd.selection_check [--seed S] [--cases N] [--mode general|shortk|midm] [MxNxK ...]
+    python -m h100_gemm_amd.selection_check [--seed S] [--cases N] [--mode general|shortk|midm]
+                                            [--write-tuned FILE] [MxNxK ...]
 """
 from __future__ import annotations
 
@@ -78,6 +79,9 @@ def main(argv=None) -> int:
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--cases", type=int, default=30, help="random shapes (0: only the shapes given)")
     ap.add_argument("--mode", default="general", choices=["general", "shortk", "midm"])
+    ap.add_argument("--write-tuned", metavar="FILE", default=None,
+                    help="append `M N K config-name` for every shape where a candidate beats the automatic "
+                         "choice by more than 2 %% (the format MI_GEMM_TUNED_FILE reads)")
     ap.add_argument("shapes", nargs="*", help="further shapes as MxNxK")
     a = ap.parse_args(argv)
     rng = np.random.default_rng(a.seed)
@@ -103,6 +107,9 @@ def main(argv=None) -> int:
         flag = f"  <-- auto loses {100 * loss:.0f} % to {mi.config_name(best)}" if loss > 0.04 else ""
         print(f"{M}x{N}x{K}: auto {mi.config_name(auto)} {t_auto * 1e3:.1f} us {flops / t_auto / 1e9:.0f} TFLOP/s; "
               f"best candidate {mi.config_name(best)} {times[best] * 1e3:.1f} us [{every}]{flag}", flush=True)
+        if a.write_tuned and loss > 0.02:
+            with open(a.write_tuned, "a") as f:
+                f.write(f"{M} {N} {K} {mi.config_name(best)}\n")
         for b in (dA, dB, dC):
             b.free()
     if losses:

@@ -90,6 +90,11 @@ const char* mi_gemm_config_name(int config);
 int mi_gemm_find_config(const char* name);
 /* The config MI_CONFIG_AUTO resolves to for this shape (never negative for valid shapes). */
 int mi_gemm_select_config(int dtype, int M, int N, int K);
+/* Number of `M N K config-name` lines loaded from the file named by the environment variable
+ * MI_GEMM_TUNED_FILE (read once, on first use; 0 without it).  MI_CONFIG_AUTO takes a listed
+ * shape's configuration instead of asking the time model -- the run-time counterpart of the
+ * tuner's persisted results (gemm_tuner.py:135-164), keyed on all of M, N, K. */
+int mi_gemm_tuned_entries(void);
 /* 1 if `config` can run this shape (alignment / divisibility rules of that kernel). */
 int mi_gemm_config_supports(int config, int dtype, int M, int N, int K);
 /* Workgroups and static LDS bytes the config launches for this shape (0 if unsupported). */

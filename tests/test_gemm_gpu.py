@@ -12,6 +12,7 @@ determinism).
 import os
 import re
 import subprocess
+import sys
 from pathlib import Path
 
 import numpy as np
@@ -372,6 +373,30 @@ def test_overflow_underflow_and_nan_follow_ieee(mi, orc, M, N, K):
     A[row, K // 2] = 0x7FC0
     C = orc.to_f32(Dev(mi, A, B, M, N).run(K))
     assert np.isnan(C[row]).all() and not np.isnan(np.delete(C, row, axis=0)).any()
+
+
+def test_tuned_shapes_file_is_used_by_the_launch(mi, orc, tmp_path):
+    """A shape listed in MI_GEMM_TUNED_FILE runs the listed configuration: in a process of its
+    own (the file is read once), the automatic launch leaves the trace records of that
+    configuration's grid and the oracle's bits."""
+    tuned = tmp_path / "tuned.txt"
+    tuned.write_text("768 1024 512 m128x128_w2x2_g4_b1_o2\n")
+    code = (
+        "import numpy as np, h100_gemm_amd as mi\n"
+        "from oracle import oracle as orc\n"
+        "M, N, K = 768, 1024, 512\n"
+        "A, B = orc.fill_randint((M, K), 69, 1), orc.fill_randint((N, K), 69, 2)\n"
+        "dA, dB, dC = mi.DeviceBuffer.from_numpy(A), mi.DeviceBuffer.from_numpy(B), mi.DeviceBuffer(M * N * 2)\n"
+        "words = mi._lib.load().mi_gemm_trace_words(M, N, K)\n"
+        "dDB = mi.DeviceBuffer(words * 4); dDB.fill_bytes(0xFF)\n"
+        "mi.runKernel(M, N, K, dA, dB, dC, dDB); mi.synchronize()\n"
+        "db = dDB.to_numpy((words,), np.int32)\n"
+        "print(mi.config_name(mi.select_config(M, N, K)), int((db[5::6] == 1).sum()),\n"
+        "      bool((dC.to_numpy((M, N), np.uint16) == orc.reference_cpu_gemm(A, B)).all()))\n")
+    env = dict(os.environ, MI_GEMM_TUNED_FILE=str(tuned), PYTHONPATH=str(ROOT))
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env, cwd=ROOT, timeout=100)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert out.stdout.split() == ["m128x128_w2x2_g4_b1_o2", "48", "True"], out.stdout     # 6 x 8 tiles of 128 x 128
 
 
 def test_output_buffer_is_not_overrun(mi, orc):

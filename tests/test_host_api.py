@@ -4,8 +4,10 @@ mirror of the reference's host functions behaves like them, the kernel configura
 is consistent, and the tile-order mapping used by the kernels is a bijection."""
 import ctypes
 import itertools
+import os
 import re
 import subprocess
+import sys
 from pathlib import Path
 
 import numpy as np
@@ -276,4 +278,31 @@ def test_selection_check_tool_is_seeded_and_knows_the_candidates():
     assert len(names) == 7 and all(n.startswith("m") for n in names)
     p = sc.bf16_pattern((5, 7), 1)
     assert p.shape == (5, 7) and p.dtype == np.uint16 and ((p & 0x7FFF) < 0x3F80).all()
+
+
+def test_tuned_shapes_file_overrides_the_model(mi, tmp_path):
+    """MI_GEMM_TUNED_FILE: `M N K config-name` lines, read once per process, consulted before
+    the time model; malformed lines, unknown names and decode configurations whose
+    preconditions the shape violates are ignored."""
+    tuned = tmp_path / "tuned.txt"
+    tuned.write_text("# shapes tuned on this machine\n"
+                     "8192 8192 8192 m256x256_w2x2_g8_b1   # not the model's choice\n"
+                     "1000 1000 1000 m256x192_w2x2_g4_b3\n"
+                     "512 512 512 no_such_config\n"
+                     "this line does not parse\n"
+                     "4096 4096 4096 k128x128_n5            # decode kernel: M too large, ignored at use\n"
+                     "64 8192 8192 s64x32_n3\n")
+    code = ("import h100_gemm_amd as mi\n"
+            "L = mi._lib.load()\n"
+            "print(L.mi_gemm_tuned_entries())\n"
+            "for s in [(8192, 8192, 8192), (1000, 1000, 1000), (512, 512, 512), (4096, 4096, 4096), (64, 8192, 8192), (8192, 8192, 4096)]:\n"
+            "    print(mi.config_name(mi.select_config(*s)))\n")
+    env = dict(os.environ, MI_GEMM_TUNED_FILE=str(tuned), PYTHONPATH=str(ROOT))
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env, cwd=ROOT)
+    assert out.returncode == 0, out.stderr
+    lines = out.stdout.split()
+    assert lines[0] == "4"                                   # four lines name a compiled configuration
+    assert lines[1:] == ["m256x256_w2x2_g8_b1", "m256x192_w2x2_g4_b3", "m128x128_w2x2_g4_b1_o2",
+                         "m256x256_w2x2_g4_b3", "s64x32_n3", "m256x256_w2x2_g4_b3"], lines
+    assert mi._lib.load().mi_gemm_tuned_entries() == 0       # this process has no such file
 
