@@ -237,9 +237,35 @@ assert all(n in {config_name(c) for c in CONFIGS} for n in TUNED_SHAPES.values()
 # N = 8192 for 8192 <= K <= 16384; the tiled kernels win for narrow B (M = 128, N <= 4096:
 # 11-20 against 14-21 us; M = 64, N = 2048: 12.5 against 14.2 us) and for very long K
 # (8192 x 28672: 97 against 105 us at M = 64, 106 against 136 us at M = 128).
-DECODE_LADDER = [(16, "s16x32_n5", "true"), (32, "s32x32_n4", "true"),
+# Measured with B rotated through enough copies to come from HBM (selection_check, decode mode):
+#  * vocabulary-wide B with a short K (N >= 32768, K <= 4096): the split-K kernel's 128-row
+#    workgroups beat the single-pass kernel's 32-row ones (32 x 32768 x 4096: 47.5 against
+#    54 us; 32 x 65536 x 4096: 93 against 106);
+#  * 32 < M <= 64 with a short K: the single-pass kernel, no second launch (64 x 8192 x 2048:
+#    10.1 against 12.8 us; 40 x 2048 x 4096: 9.5 against 11.4; level with split-K from K = 8192),
+#    but not for wide B (64 x 28672 x 1024: 24.8 against 14.5 us for split-K);
+#  * 64 < M <= 128, N = 8192: 128x256 tiles from K = 10240 (12288: 50-53 against 54-62 us;
+#    20480: 73-77 against 87-98), except where the row pitch is a power of two (16384: 79-82
+#    against 61-68 us: the tiled kernels' rows then start in the same few memory channels).
+#  * narrow B with a long K at M <= 32 (N < 4096: fewer 32-row workgroups than CUs, each
+#    walking all of K alone) from K = 12288: split-K spreads K over the idle CUs (21 x 1792 x
+#    12288: 16.7 against 27.3 us; 32 x 2048 x 28672: 32 against 70; at K = 8192 the single pass
+#    is still ahead, 8 x 1024 x 8192: 10.3 against 15.1);
+#  * 64 < M <= 128: the split-K decode kernel from N = 12288 (74 x 14336 x 5120: 38 against
+#    42 us; 81 x 15360 x 6848: 47 against 55).
+#  * the single-pass kernel runs N / 32 workgroups, best when they fill whole rounds of the 256
+#    CUs (N = 8192, 16384): at N = 4096, 5120, 9216, 10240, 12288, 18432 (under 80 % of the
+#    last round's CUs busy) split-K is 5-30 % ahead once B is large enough to hide its
+#    second launch (32 x 5120 x 12288: 28.5 against 35.3 us; 13 x 10240 x 16384: 63 against 70;
+#    32 x 12288 x 8192: 40 against 44; but 32 x 4096 x 4096: 14 against 10.6).
+_STREAM_ROUNDS_UNDER_80 = "((N + 31) / 32) * 5 < ((((N + 31) / 32) + 255) / 256) * 1024"
+DECODE_LADDER = [(32, "k64x128_n6", "(N >= 32768 && K <= 4096) || (N < 4096 && K >= 12288) || "
+                                    "(" + _STREAM_ROUNDS_UNDER_80 + " && (long long)N * K >= 50331648LL)"),
+                 (16, "s16x32_n5", "true"), (32, "s32x32_n4", "true"),
+                 (64, "s64x32_n3", "N <= 12288 && (K <= 4096 || (N >= 4096 && K <= 6144))"),
                  (64, "k64x128_n6", "N >= 4096 && K < 24576"),
-                 (128, "k128x128_n5", "N >= 16384 || (N >= 8192 && K >= 8192 && K < 24576)"),
+                 (128, "m128x256_w2x2_g4_b1", "N >= 4096 && N < 12288 && K >= 10240 && K < 24576 && (K & (K - 1)) != 0"),
+                 (128, "k128x128_n5", "N >= 12288 || (N >= 8192 && K >= 8192 && K < 24576)"),
                  # very long K: 128x256 tiles (one row of tiles covers M, B is read once) in split-K
                  # pieces: 97 / 106 us at M = 64 / 128 against 105 / 136 us for the decode kernels
                  # and 115-143 us for the other tiles, between which the time model cannot tell

@@ -8,7 +8,7 @@ against the best candidate and every candidate's time.  A tuning aid for the con
 (``gemm_tuner.py:82-133``) for the choice between compiled kernels instead of between
 template parameters.
 
-    python -m h100_gemm_amd.selection_check [--seed S] [--cases N] [--mode general|shortk|midm]
+    python -m h100_gemm_amd.selection_check [--seed S] [--cases N] [--mode general|shortk|midm|decode]
                                             [--write-tuned FILE] [MxNxK ...]
 """
 from __future__ import annotations
@@ -22,9 +22,10 @@ import h100_gemm_amd as mi
 from h100_gemm_amd import kernel_configs as kc
 
 
-def candidates() -> list[int]:
-    """indices of the configurations the time model chooses from (those with a measured EFF)"""
-    return [i for i, c in enumerate(kc.CONFIGS) if c.get("EFF")]
+def candidates(decode: bool = False) -> list[int]:
+    """indices of the configurations the time model chooses from (those with a measured EFF);
+    with `decode` also the decode kernels of the ladder in front of the model"""
+    return [i for i, c in enumerate(kc.CONFIGS) if c.get("EFF") or (decode and c["KIND"] in ("stream", "skinny"))]
 
 
 def random_shape(rng: np.random.Generator, it: int, mode: str) -> tuple[int, int, int]:
@@ -37,6 +38,10 @@ def random_shape(rng: np.random.Generator, it: int, mode: str) -> tuple[int, int
         M, N, K = 64 * rng.integers(2, 120), 64 * rng.integers(2, 120), 8 * rng.integers(32, 1000)
     if mode == "shortk":
         K = rng.choice([128 * rng.integers(1, 13), rng.integers(64, 1600), 64 * rng.integers(1, 24)])
+    elif mode == "decode":
+        M = rng.choice([rng.integers(1, 33), rng.integers(33, 129), 16 * rng.integers(1, 9)])
+        N = rng.choice([256 * rng.integers(1, 33), 4 * rng.integers(64, 2048), 1024 * rng.integers(1, 29)])
+        K = rng.choice([64 * rng.integers(8, 257), 1024 * rng.integers(1, 29)])
     elif mode == "midm":
         M = rng.choice([rng.integers(129, 1500), 64 * rng.integers(3, 24)])
         N = rng.choice([256 * rng.integers(4, 33), rng.integers(1024, 8192)])
@@ -58,17 +63,18 @@ def bf16_pattern(shape, seed: int) -> np.ndarray:
     return np.resize(block, shape)
 
 
-def time_config(config: int, params, launches: int) -> float:
-    """best of three batches of back-to-back launches, milliseconds per launch"""
-    for _ in range(max(3, launches // 4)):
-        mi.gpu_gemm(params, config=config)
+def time_config(config: int, params: list, launches: int) -> float:
+    """best of three batches of back-to-back launches, milliseconds per launch; `params` holds
+    one GemmParams per copy of B and the launches go round them"""
+    for i in range(max(3, launches // 4)):
+        mi.gpu_gemm(params[i % len(params)], config=config)
     mi.synchronize()
     best = float("inf")
     for _ in range(3):
         timer = mi.GPUTimer()
         timer.tick()
-        for _ in range(launches):
-            mi.gpu_gemm(params, config=config)
+        for i in range(launches):
+            mi.gpu_gemm(params[i % len(params)], config=config)
         timer.tick()
         best = min(best, timer.report_last_ms() / launches)
     return best
@@ -78,7 +84,7 @@ def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--cases", type=int, default=30, help="random shapes (0: only the shapes given)")
-    ap.add_argument("--mode", default="general", choices=["general", "shortk", "midm"])
+    ap.add_argument("--mode", default="general", choices=["general", "shortk", "midm", "decode"])
     ap.add_argument("--write-tuned", metavar="FILE", default=None,
                     help="append `M N K config-name` for every shape where a candidate beats the automatic "
                          "choice by more than 2 %% (the format MI_GEMM_TUNED_FILE reads)")
@@ -88,12 +94,16 @@ def main(argv=None) -> int:
     shapes = [random_shape(rng, it, a.mode) for it in range(a.cases)]
     shapes += [tuple(int(v) for v in s.split("x")) for s in a.shapes]
     lib = mi._lib.load()
-    cands = candidates()
+    cands = candidates(decode=a.mode == "decode")
     losses = []
     for M, N, K in shapes:
         A, B = bf16_pattern((M, K), 1), bf16_pattern((N, K), 2)
-        dA, dB, dC = mi.DeviceBuffer.from_numpy(A), mi.DeviceBuffer.from_numpy(B), mi.DeviceBuffer(M * N * 2)
-        params = mi.GemmParams(M, N, K, dA, dB, dC)
+        # decode shapes stream B from HBM in their real use (many layers of weights): enough
+        # copies of B to exceed the 256 MB memory-side cache, visited in turn
+        copies = min(8, -(-(600 << 20) // B.nbytes)) if M <= 128 else 1
+        dA, dC = mi.DeviceBuffer.from_numpy(A), mi.DeviceBuffer(M * N * 2)
+        dBs = [mi.DeviceBuffer.from_numpy(B) for _ in range(copies)]
+        params = [mi.GemmParams(M, N, K, dA, dB, dC) for dB in dBs]
         flops = 2.0 * M * N * K
         launches = int(min(200, max(10, 3e-2 / (flops / 1.2e15 + 5e-6))))     # ~30 ms per batch
         auto = mi.select_config(M, N, K)
@@ -110,7 +120,7 @@ def main(argv=None) -> int:
         if a.write_tuned and loss > 0.02:
             with open(a.write_tuned, "a") as f:
                 f.write(f"{M} {N} {K} {mi.config_name(best)}\n")
-        for b in (dA, dB, dC):
+        for b in [dA, dC] + dBs:
             b.free()
     if losses:
         print(f"{len(losses)} shapes: mean loss against the best candidate {100 * float(np.mean(losses)):.2f} %, "

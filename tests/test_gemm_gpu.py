@@ -725,7 +725,8 @@ def test_automatic_choice_across_regimes_bit_exact(mi, orc):
     for M in (1, 16, 17, 32, 33, 64, 65, 128, 129, 256, 257):
         shapes += [(M, 4096, 4096), (M, 1024, 8192), (M, 8192, 512), (M, 4100, 1088)]
     shapes += [(64, 4096, 24576), (128, 4096, 24576), (96, 16384, 1024), (128, 8192, 8192), (48, 8192, 2048),
-               (130, 4096, 24640), (512, 512, 4096), (3000, 3000, 264), (384, 384, 6016), (192, 8192, 2048)]
+               (130, 4096, 24640), (512, 512, 4096), (3000, 3000, 264), (384, 384, 6016), (192, 8192, 2048),
+               (64, 8192, 8192), (24, 32768, 2048), (96, 8192, 12288), (96, 8192, 16384), (40, 8192, 6144)]
     seen = set()
     for M, N, K in shapes:
         cfg = mi.select_config(M, N, K)
@@ -733,5 +734,5 @@ def test_automatic_choice_across_regimes_bit_exact(mi, orc):
         print(f"case M={M} N={N} K={K} -> {mi.config_name(cfg)} grid {mi.config_grid(cfg, M, N, K)}", flush=True)
         check(mi, orc, M, N, K, "int", exact=True)
     # the sweep is only worth its time if it reaches the different kernel families
-    assert {"s16x32_n5", "s32x32_n4", "k64x128_n6", "k128x128_n5"} <= seen, seen
+    assert {"s16x32_n5", "s32x32_n4", "s64x32_n3", "k64x128_n6", "k128x128_n5"} <= seen, seen
     assert any(n.startswith("m128x256") for n in seen) and any(n.startswith("m128x128") for n in seen), seen
