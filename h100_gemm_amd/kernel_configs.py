@@ -263,8 +263,12 @@ DECODE_LADDER = [(32, "k64x128_n6", "(N >= 32768 && K <= 4096) || (N < 4096 && K
                                     "(" + _STREAM_ROUNDS_UNDER_80 + " && (long long)N * K >= 50331648LL)"),
                  (16, "s16x32_n5", "true"), (32, "s32x32_n4", "true"),
                  (64, "s64x32_n3", "N <= 12288 && (K <= 4096 || (N >= 4096 && K <= 6144))"),
-                 (64, "k64x128_n6", "N >= 4096 && K < 24576"),
+                 # (also for 32 < M <= 64: 48 x 6584 x 15360 45 against 56 us, 47 x 6144 x 23552 63 against 70)
                  (128, "m128x256_w2x2_g4_b1", "N >= 4096 && N < 12288 && K >= 10240 && K < 24576 && (K & (K - 1)) != 0"),
+                 # (narrower B with a long K: 64 x 3328 x 15808 29.4 against 32.4 us tiled, 80 x 2104 x 18432
+                 # 27.2 against 29.0, 96 x 3636 x 23552 51 against 55.5)
+                 (64, "k64x128_n6", "(N >= 4096 && K < 24576) || (N >= 2048 && N < 4096 && K >= 12288 && K < 24576)"),
+                 (128, "k128x128_n5", "N >= 2048 && N < 4096 && K >= 12288"),
                  (128, "k128x128_n5", "N >= 12288 || (N >= 8192 && K >= 8192 && K < 24576)"),
                  # very long K: 128x256 tiles (one row of tiles covers M, B is read once) in split-K
                  # pieces: 97 / 106 us at M = 64 / 128 against 105 / 136 us for the decode kernels
