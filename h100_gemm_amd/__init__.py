@@ -23,7 +23,7 @@ from . import _lib
 from ._lib import (MI_C_COL_MAJOR, MI_C_ROW_MAJOR, MI_CONFIG_AUTO, MI_DTYPE_BF16, MI_DTYPE_FP16, DeviceProps,
                    MiGemmError)
 
-__all__ = ["runKernel", "run_kernel", "gpu_gemm", "gemm_epilogue", "MI_C_ROW_MAJOR", "MI_C_COL_MAJOR", "reference_gpu_gemm", "GemmParams", "DeviceBuffer", "GPUTimer",
+__all__ = ["runKernel", "run_kernel", "gpu_gemm", "gemm_epilogue", "workspace_bytes", "MI_C_ROW_MAJOR", "MI_C_COL_MAJOR", "reference_gpu_gemm", "GemmParams", "DeviceBuffer", "GPUTimer",
            "device_props", "num_configs", "config_name", "find_config", "select_config",
            "config_grid", "synchronize", "MiGemmError", "MI_CONFIG_AUTO", "MI_DTYPE_BF16",
            "MI_DTYPE_FP16"]
@@ -102,14 +102,29 @@ def _config_index(L, config) -> int:
 
 
 def gemm_epilogue(params: GemmParams, config: int | str = MI_CONFIG_AUTO, dtype: int = MI_DTYPE_BF16,
-                  c_layout: int = MI_C_ROW_MAJOR, stream=None) -> None:
+                  c_layout: int = MI_C_ROW_MAJOR, stream=None, workspace: "DeviceBuffer | None" = None) -> None:
     """The GEMM with the golden's epilogue, C = (CType)(acc * alpha + beta) with beta a plain
     scalar (reference.h:40), and C row-major or column-major (C[n*M + m], the layout the
-    reference's bf16 kernel writes, matmul_utils.cuh:529,545)."""
+    reference's bf16 kernel writes, matmul_utils.cuh:529,545).  With ``workspace`` (a
+    DeviceBuffer of at least ``workspace_bytes(...)`` bytes) split-K partial sums go there and
+    the call allocates nothing, like the reference's launcher (matmul_h100_optimal.cu:32-59)."""
     L = _lib.load()
+    if workspace is not None:
+        _lib.check(L.mi_gemm_epilogue_ws(_config_index(L, config), dtype, params.M, params.N, params.K,
+                                         _ptr(params.A), _ptr(params.B), _ptr(params.C), params.alpha,
+                                         params.beta, c_layout, workspace.ptr, workspace.nbytes,
+                                         _stream(stream)))
+        return
     _lib.check(L.mi_gemm_epilogue(_config_index(L, config), dtype, params.M, params.N, params.K,
                                   _ptr(params.A), _ptr(params.B), _ptr(params.C), params.alpha,
                                   params.beta, c_layout, _stream(stream)))
+
+
+def workspace_bytes(M: int, N: int, K: int, config: int | str = MI_CONFIG_AUTO, dtype: int = MI_DTYPE_BF16,
+                    c_layout: int = MI_C_ROW_MAJOR) -> int:
+    """Bytes of split-K workspace the library's kernel choice wants for this shape (0: none)."""
+    L = _lib.load()
+    return int(L.mi_gemm_workspace_bytes(_config_index(L, config), dtype, M, N, K, c_layout))
 
 
 def reference_gpu_gemm(params: GemmParams, dtype: int = MI_DTYPE_BF16, stream=None) -> None:

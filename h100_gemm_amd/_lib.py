@@ -42,6 +42,10 @@ SYMBOLS = {
                              C.c_void_p, C.c_void_p, C.c_void_p]),
     "mi_gemm_epilogue": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
                                    C.c_void_p, C.c_float, C.c_float, C.c_int, C.c_void_p]),
+    "mi_gemm_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]),
+    "mi_gemm_epilogue_ws": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
+                                      C.c_void_p, C.c_float, C.c_float, C.c_int, C.c_void_p, C.c_size_t,
+                                      C.c_void_p]),
     "mi_reference_gpu_gemm": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
                                         C.c_void_p, C.c_float, C.c_float, C.c_void_p]),
     "mi_gemm_num_configs": (C.c_int, []),

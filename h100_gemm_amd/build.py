@@ -112,12 +112,35 @@ def build(jobs: int | None = None, force: bool = False, verbose: bool = True) ->
     return LIB
 
 
+# Two points of the tuner's search space, rendered from template/matmul_mi355x.hip.jinja and
+# compiled as standalone `./test` programs -- the tuner's own flow (render -> hipcc -> run),
+# whose programs instantiate the kernels directly instead of going through the library's
+# dispatch.  Built here, where hipcc runs without a GPU, so that the GPU tests only run them.
+TUNER_SAMPLES = PKG / "harness" / "tuner_samples"
+TUNER_SAMPLE_CONFIGS = [
+    dict(KIND="mfma16", BM=256, BN=256, WM=2, WN=2, NS=4, SWZ=1, GROUP=4, DTL=1, EPI=1, DRAIN=3, OCC=1),
+    dict(KIND="tile", BM=128, BN=128, WM=2, WN=2, NS=4, SWZ=1, GROUP=8, DTL=1, EPI=1, DRAIN=0, OCC=2),
+]
+
+
+def build_tuner_samples(jobs: int = 2, verbose: bool = True) -> Path:
+    from .gemm_tuner import GemmTuner
+    tuner = GemmTuner(output_dir=str(TUNER_SAMPLES), only=TUNER_SAMPLE_CONFIGS)
+    built = tuner.prebuild(jobs)
+    if len(built) != len(TUNER_SAMPLE_CONFIGS) or not all(built.values()):
+        raise RuntimeError(f"tuner sample programs failed to compile: {built}")
+    if verbose:
+        print(f"built {len(built)} tuner sample programs in {tuner.bin_dir}")
+    return tuner.bin_dir
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__)
     ap.add_argument("-j", "--jobs", type=int, default=None)
     ap.add_argument("--force", action="store_true")
     a = ap.parse_args(argv)
     build(a.jobs, a.force)
+    build_tuner_samples()
     return 0
 
 

@@ -101,14 +101,36 @@ int choose_tile_splits(const mi::KernelEntry& e, int M, int N, int K, bool split
     return mi::best_splits(e, M, N, K, true, ptr_aligned, cus, k_per_split, nullptr);
 }
 
-// fp32 partial-sum workspace of the split-K kernels: one buffer per device, grown on
-// demand.  Launches that use it are ordered on their stream; callers that run split-K
-// launches on several streams of one device at once must serialise them.  Workspace and
-// CU count belong to the device that is current when the call is made.
+// ---- where the split-K kernels put their fp32 partial sums ----------------------------
+// Two sources, chosen by the entry point:
+//  * LIBRARY (mi_gemm_bf16 / _ex / _epilogue): one buffer per (device, stream), allocated on
+//    first use and replaced by a larger one on demand.  A buffer is never freed while the
+//    process lives: launches already enqueued and captured graphs keep its address, so a
+//    replaced buffer only moves to a retired list (sizes are powers of two, so the retired
+//    ones together stay below the live one).  Launches on one stream are ordered and
+//    launches on different streams use different buffers, so concurrent split-K calls do
+//    not meet.  A stream that is being captured cannot allocate: if it has no buffer that is
+//    large enough yet, the launch runs unsplit instead.
+//  * CALLER (mi_gemm_epilogue_ws): the caller's buffer, nothing is allocated; too small (or
+//    NULL) means the launch runs unsplit.
+// The kernels overwrite every partial they later read ([piece][M][N], all of it), so no
+// buffer needs clearing between calls.
 constexpr int kMaxDevices = 64;
+
+enum WsMode { WS_LIBRARY, WS_CALLER };
+struct WsSource {
+    WsMode mode = WS_LIBRARY;
+    void* ptr = nullptr;      // WS_CALLER: the caller's buffer
+    size_t bytes = 0;
+};
+struct StreamWs {
+    hipStream_t stream;
+    float* ptr;
+    size_t bytes;
+};
 struct DeviceState {
-    float* ws = nullptr;
-    size_t ws_bytes = 0;
+    std::vector<StreamWs> ws;        // live buffers, one per stream that ran a split-K launch
+    std::vector<void*> retired;      // replaced buffers: kept until the process ends
     int cus = 0;
 };
 std::mutex g_ws_mutex;
@@ -120,23 +142,45 @@ DeviceState& device_state() {
     return g_dev[dev];
 }
 
-hipError_t ensure_workspace(size_t bytes, float** out) {
+// 0: *out holds `bytes` of workspace; 1: none to be had without allocating where that is not
+// possible (the caller runs the launch unsplit); < 0: MI_ERR_* with the message set.
+int acquire_workspace(const WsSource& src, size_t bytes, hipStream_t stream, float** out) {
+    *out = nullptr;
+    if (src.mode == WS_CALLER) {
+        if (!src.ptr || src.bytes < bytes) return 1;
+        *out = (float*)src.ptr;
+        return 0;
+    }
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     DeviceState& st = device_state();
-    if (bytes > st.ws_bytes) {
-        if (st.ws) {
-            hipError_t e = hipFree(st.ws);     // waits for work that may still use it
-            st.ws = nullptr;
-            st.ws_bytes = 0;
-            if (e != hipSuccess) return e;
-        }
-        const size_t want = bytes < (size_t)(32u << 20) ? (size_t)(32u << 20) : bytes;
-        hipError_t e = hipMalloc((void**)&st.ws, want);
-        if (e != hipSuccess) return e;
-        st.ws_bytes = want;
+    StreamWs* mine = nullptr;
+    for (StreamWs& w : st.ws)
+        if (w.stream == stream) mine = &w;
+    if (mine && mine->bytes >= bytes) {
+        *out = mine->ptr;
+        return 0;
     }
-    *out = st.ws;
-    return hipSuccess;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) != hipSuccess) {
+        (void)hipGetLastError();
+        return 1;      // e.g. the null stream while another stream captures: do not allocate
+    }
+    if (cap != hipStreamCaptureStatusNone) return 1;
+    size_t want = (size_t)4 << 20;
+    while (want < bytes) want <<= 1;
+    float* p = nullptr;
+    hipError_t e = hipMalloc((void**)&p, want);
+    if (e != hipSuccess)
+        return fail(MI_ERR_HIP, "split-K workspace allocation of %zu bytes failed: %s", want, hipGetErrorString(e));
+    if (mine) {
+        st.retired.push_back(mine->ptr);
+        mine->ptr = p;
+        mine->bytes = want;
+    } else {
+        st.ws.push_back({stream, p, want});
+    }
+    *out = p;
+    return 0;
 }
 
 int compute_units() {
@@ -228,6 +272,24 @@ struct Choice {
     int M, N, K, flags, requested, cus;   // key; requested = the caller's config (MI_CONFIG_AUTO or an index)
     int config, splits, k_per_split;
 };
+Choice compute_choice(int requested, int M, int N, int K, bool streamable, bool splittable, bool ptr_aligned) {
+    const int flags = (streamable ? 1 : 0) | (splittable ? 2 : 0) | (ptr_aligned ? 4 : 0);
+    const int cus = compute_units();
+    Choice c{M, N, K, flags, requested, cus, requested, 1, K};
+    if (requested == MI_CONFIG_AUTO) {
+        c.config = tuned_config(M, N, K, streamable);
+        if (c.config < 0) c.config = mi::select_kernel(M, N, K, streamable, splittable, ptr_aligned, cus);
+    }
+    const mi::KernelEntry& e = mi::kKernels[c.config];
+    if (e.kind == mi::KIND_MFMA16) {
+        c.splits = choose_tile_splits(e, M, N, K, splittable, ptr_aligned, cus, &c.k_per_split);
+    } else if (e.kind == mi::KIND_SKINNY && streamable && M <= e.BM) {
+        const int tiles_n = (N + e.BN - 1) / e.BN;
+        c.splits = choose_splits(tiles_n, K, cus, e.lds_bytes, e.BM);   // <= K / 64: no empty split
+        c.k_per_split = ((K / 64 + c.splits - 1) / c.splits) * 64;
+    }
+    return c;
+}
 Choice choose(int requested, int M, int N, int K, bool streamable, bool splittable, bool ptr_aligned) {
     static thread_local Choice memo[4] = {};
     static thread_local int next = 0;
@@ -237,14 +299,7 @@ Choice choose(int requested, int M, int N, int K, bool streamable, bool splittab
         if (c.M == M && c.N == N && c.K == K && c.flags == flags && c.requested == requested && c.cus == cus &&
             c.splits > 0)
             return c;
-    Choice c{M, N, K, flags, requested, cus, requested, 1, K};
-    if (requested == MI_CONFIG_AUTO) {
-        c.config = tuned_config(M, N, K, streamable);
-        if (c.config < 0) c.config = mi::select_kernel(M, N, K, streamable, splittable, ptr_aligned, cus);
-    }
-    const mi::KernelEntry& e = mi::kKernels[c.config];
-    if (e.kind == mi::KIND_MFMA16)
-        c.splits = choose_tile_splits(e, M, N, K, splittable, ptr_aligned, cus, &c.k_per_split);
+    const Choice c = compute_choice(requested, M, N, K, streamable, splittable, ptr_aligned);
     memo[next] = c;
     next = (next + 1) & 3;
     return c;
@@ -252,7 +307,7 @@ Choice choose(int requested, int M, int N, int K, bool streamable, bool splittab
 
 // One GEMM launch (two for split-K): argument checks, kernel choice, aligned / predicated twin.
 int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const void* B, void* C,
-             int* DB, float alpha, float beta, void* stream) {
+             int* DB, float alpha, float beta, void* stream, const WsSource& wsrc = WsSource{}) {
     int rc = check_args(config, dtype, M, N, K, A, B, C);
     if (rc != MI_OK) return rc;
     const bool streamable = shape_is_streamable(M, N, K, A, B, C);
@@ -296,13 +351,15 @@ int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const vo
             return fail(MI_ERR_UNSUPPORTED,
                         "config %s needs M <= %d, N %% 4 == 0, K %% 64 == 0 and 16-byte aligned operands",
                         e.name, e.BM);
-        const int tiles_n = (N + e.BN - 1) / e.BN;
-        args.splits = choose_splits(tiles_n, K, compute_units(), e.lds_bytes, e.BM);   // <= K / 64: no empty split
-        args.k_per_split = ((K / 64 + args.splits - 1) / args.splits) * 64;
+        args.splits = choice.splits;
+        args.k_per_split = choice.k_per_split;
         if (args.splits > 1) {
-            hipError_t we = ensure_workspace((size_t)args.splits * M * N * sizeof(float), &args.ws);
-            if (we != hipSuccess)
-                return fail(MI_ERR_HIP, "split-K workspace allocation failed: %s", hipGetErrorString(we));
+            const int wrc = acquire_workspace(wsrc, (size_t)args.splits * M * N * sizeof(float), (hipStream_t)stream, &args.ws);
+            if (wrc < 0) return wrc;
+            if (wrc > 0) {           // no workspace to be had: one pass over all of K
+                args.splits = 1;
+                args.k_per_split = K;
+            }
         }
         hipError_t err = e.launch[dtype][0](args, (hipStream_t)stream);
         if (err != hipSuccess)
@@ -318,9 +375,12 @@ int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const vo
         args.splits = choice.splits;
         args.k_per_split = choice.k_per_split;
         if (args.splits > 1) {
-            hipError_t we = ensure_workspace((size_t)args.splits * M * N * sizeof(float), &args.ws);
-            if (we != hipSuccess)
-                return fail(MI_ERR_HIP, "split-K workspace allocation failed: %s", hipGetErrorString(we));
+            const int wrc = acquire_workspace(wsrc, (size_t)args.splits * M * N * sizeof(float), (hipStream_t)stream, &args.ws);
+            if (wrc < 0) return wrc;
+            if (wrc > 0) {
+                args.splits = 1;
+                args.k_per_split = K;
+            }
         }
     }
     hipError_t err = fn(args, (hipStream_t)stream);
@@ -436,6 +496,44 @@ int mi_gemm_epilogue(int config, int dtype, int M, int N, int K, const void* A, 
 int mi_gemm_bf16(int M, int N, int K, const uint16_t* A, const uint16_t* B, uint16_t* C, int* DB,
                  void* stream) {
     return mi_gemm_ex(MI_CONFIG_AUTO, MI_DTYPE_BF16, M, N, K, A, B, C, DB, stream);
+}
+
+size_t mi_gemm_workspace_bytes(int config, int dtype, int M, int N, int K, int c_layout) {
+    if (dtype != MI_DTYPE_BF16 && dtype != MI_DTYPE_FP16) return 0;
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    if (config != MI_CONFIG_AUTO && (config < 0 || config >= mi::kNumKernels)) return 0;
+    if ((long long)M * N > 0x7fffffffLL) return 0;
+    if (c_layout == MI_C_COL_MAJOR) {
+        const int t = M;
+        M = N;
+        N = t;
+    }
+    // The choice also depends on the alignment of the pointers, unknown here: the largest
+    // need over the cases a launch can meet.
+    size_t need = 0;
+    const bool can_stream = N % 4 == 0 && K % 64 == 0;
+    for (int aligned = 0; aligned < 2; ++aligned)
+        for (int streamable = 0; streamable < (can_stream && aligned ? 2 : 1); ++streamable) {
+            const Choice c = compute_choice(config, M, N, K, streamable != 0, N % 4 == 0, aligned != 0);
+            const size_t b = c.splits > 1 ? (size_t)c.splits * M * N * sizeof(float) : 0;
+            if (b > need) need = b;
+        }
+    return need;
+}
+
+int mi_gemm_epilogue_ws(int config, int dtype, int M, int N, int K, const void* A, const void* B, void* C,
+                        float alpha, float beta, int c_layout, void* ws, size_t ws_bytes, void* stream) {
+    if (c_layout != MI_C_ROW_MAJOR && c_layout != MI_C_COL_MAJOR)
+        return fail(MI_ERR_INVALID, "unknown C layout %d", c_layout);
+    if (!(alpha == alpha) || !(beta == beta)) return fail(MI_ERR_INVALID, "alpha or beta is NaN");
+    if (ws && !aligned16(ws)) return fail(MI_ERR_INVALID, "the workspace must be 16-byte aligned");
+    WsSource src;
+    src.mode = WS_CALLER;
+    src.ptr = ws;
+    src.bytes = ws ? ws_bytes : 0;
+    if (c_layout == MI_C_COL_MAJOR)
+        return run_gemm(config, dtype, N, M, K, B, A, C, nullptr, alpha, beta, stream, src);
+    return run_gemm(config, dtype, M, N, K, A, B, C, nullptr, alpha, beta, stream, src);
 }
 
 int mi_reference_gpu_gemm(int dtype, int M, int N, int K, const void* A, const void* B, void* C,

@@ -60,7 +60,8 @@ class GemmTuner:
     def __init__(self, template_file: str = str(DEFAULT_TEMPLATE), output_dir: str = "tuning_results",
                  work_dir: Optional[str] = None, compile_command=default_compile_command,
                  bench_args=("M", "5120", "N", "5120", "K", "4096"), timeout: float = 30.0,
-                 resume_from: Optional[str] = None):
+                 resume_from: Optional[str] = None, bin_dir: Optional[str] = None,
+                 only: Optional[List[Dict[str, int]]] = None):
         self.output_dir = Path(output_dir)
         self.output_dir.mkdir(parents=True, exist_ok=True)
         self.work_dir = Path(work_dir) if work_dir else self.output_dir
@@ -68,6 +69,10 @@ class GemmTuner:
         self.compile_command = compile_command
         self.bench_args = list(bench_args)
         self.timeout = timeout
+        # where prebuild() puts the programs and tune(prebuilt=True) looks for them
+        self.bin_dir = Path(bin_dir) if bin_dir else self.output_dir / 'bin'
+        # an explicit list of configurations instead of the grid below
+        self.only = only
 
         # Define parameter search space
         self.param_space = {
@@ -127,7 +132,7 @@ class GemmTuner:
     def benchmark_configuration(self, params: Dict[str, int], prebuilt: bool = False) -> Tuple[float, bool]:
         """Benchmark a single configuration. Returns (runtime, success)"""
         if prebuilt:
-            exe = self.output_dir / 'bin' / self.config_name(params)
+            exe = self.bin_dir / self.config_name(params)
             if not exe.exists():
                 print(f"Compilation failed for parameters: {params}")
                 return float('inf'), False
@@ -170,16 +175,18 @@ class GemmTuner:
             return False
 
     def configurations(self) -> List[Dict[str, int]]:
+        if self.only is not None:
+            return [p for p in self.only if self.is_valid_configuration(p)]
         combos = [dict(zip(self.param_space.keys(), values))
                   for values in itertools.product(*self.param_space.values())]
         return [p for p in combos if self.is_valid_configuration(p)]
 
     def prebuild(self, jobs: int = 8) -> Dict[str, bool]:
         """Render and compile every valid configuration into <output_dir>/bin."""
-        bindir = self.output_dir / 'bin'
+        bindir = self.bin_dir
         srcdir = self.output_dir / 'src'
-        bindir.mkdir(exist_ok=True)
-        srcdir.mkdir(exist_ok=True)
+        bindir.mkdir(parents=True, exist_ok=True)
+        srcdir.mkdir(parents=True, exist_ok=True)
 
         def one(params):
             name = self.config_name(params)
@@ -193,94 +200,61 @@ class GemmTuner:
         with ThreadPoolExecutor(max_workers=jobs) as ex:
             return dict(ex.map(one, self.configurations()))
 
+    # ---- the sweep ----------------------------------------------------------------------
+
+    def _measure(self, params: Dict[str, int], prebuilt: bool) -> Tuple[Optional[float], bool]:
+        """(runtime in ms or None, success) of one configuration; resumed results are reused."""
+        old = self.previous.get(self.config_key(params))
+        if old is not None:
+            print("(taken from the resumed results)")
+            return (old['runtime'] if old['success'] else None), bool(old['success'])
+        runtime, ok = self.benchmark_configuration(params, prebuilt=prebuilt)
+        return (runtime if ok else None), ok
+
     def tune(self, prebuilt: bool = False):
-        """Run the tuning process and save results"""
-        results = []
-        best_runtime = float('inf')
-        best_params = None
+        """Time every valid configuration; returns (best_params, best_runtime, results).
 
-        # Generate all parameter combinations
-        param_combinations = [dict(zip(self.param_space.keys(), values))
-                              for values in itertools.product(*self.param_space.values())]
-
-        total_configs = len([p for p in param_combinations if self.is_valid_configuration(p)])
-        tested_configs = 0
-
-        for params in param_combinations:
-            if not self.is_valid_configuration(params):
-                continue
-
-            tested_configs += 1
-            print(f"\nTesting configuration {tested_configs}/{total_configs}:")
+        A configuration that fails to compile, exits non-zero, prints no latency line or runs
+        out of time is recorded with success = False and the sweep goes on
+        (gemm_tuner.py:49-72).  After each one the results JSON and the summary are rewritten
+        and, when it is the fastest so far, its rendered source is kept as
+        best_matmul_mi355x.hip (gemm_tuner.py:117-133)."""
+        todo = self.configurations()
+        results: List[Dict] = []
+        best: Tuple[float, Optional[Dict[str, int]]] = (float('inf'), None)
+        for n, params in enumerate(todo, 1):
+            print(f"\nTesting configuration {n}/{len(todo)}:")
             print(params)
-
-            prev = self.previous.get(self.config_key(params))
-            if prev is not None:
-                runtime = prev['runtime'] if prev['success'] else float('inf')
-                success = prev['success']
-                print("(taken from the resumed results)")
-            else:
-                runtime, success = self.benchmark_configuration(params, prebuilt=prebuilt)
-
-            result = {
-                'params': params,
-                'runtime': runtime if success else None,
-                'success': success,
-                'timestamp': datetime.now().isoformat()
-            }
-            results.append(result)
-
-            if success:
+            runtime, ok = self._measure(params, prebuilt)
+            results.append({'params': params, 'runtime': runtime, 'success': ok,
+                            'timestamp': datetime.now().isoformat()})
+            if ok:
                 print(f"Runtime: {runtime:.4f} ms")
+                if runtime < best[0]:
+                    best = (runtime, params)
+                    print(f"New best runtime: {runtime:.4f} ms")
+                    (self.output_dir / 'best_matmul_mi355x.hip').write_text(self.generate_code(params))
+            self.save_results(results, best[1], best[0])
+        return best[1], best[0], results
 
-            if success and runtime < best_runtime:
-                best_runtime = runtime
-                best_params = params
-                print(f"New best runtime: {best_runtime:.4f} ms")
+    def save_results(self, results: List[Dict], best_params: Optional[Dict[str, int]], best_runtime: float):
+        """tuning_results_<timestamp>.json and tuning_summary.txt in the reference's formats
+        (gemm_tuner.py:135-164): the JSON holds every result, the summary the best
+        configuration followed by all successful ones, fastest first."""
+        stamp = datetime.now().strftime('%Y%m%d_%H%M%S')
+        doc = {'results': results, 'best_params': best_params, 'best_runtime': best_runtime, 'timestamp': stamp}
+        (self.output_dir / f'tuning_results_{stamp}.json').write_text(json.dumps(doc, indent=2))
 
-                # Save the best configuration immediately
-                best_config_file = self.output_dir / 'best_matmul_mi355x.hip'
-                with open(best_config_file, 'w') as f:
-                    f.write(self.generate_code(best_params))
+        def block(params):
+            return [f"{k}: {v}" for k, v in params.items()]
 
-            # Save intermediate results
-            self.save_results(results, best_params, best_runtime)
-
-        return best_params, best_runtime, results
-
-    def save_results(self, results: List[Dict], best_params: Dict[str, int], best_runtime: float):
-        """Save results to disk"""
-        timestamp = datetime.now().strftime('%Y%m%d_%H%M%S')
-
-        # Save detailed results
-        results_file = self.output_dir / f'tuning_results_{timestamp}.json'
-        with open(results_file, 'w') as f:
-            json.dump({
-                'results': results,
-                'best_params': best_params,
-                'best_runtime': best_runtime,
-                'timestamp': timestamp
-            }, f, indent=2)
-
-        # Save summary
-        summary_file = self.output_dir / 'tuning_summary.txt'
-        with open(summary_file, 'w') as f:
-            f.write(f"Tuning completed at: {timestamp}\n")
-            f.write(f"Best runtime: {best_runtime:.4f} ms\n")
-            if best_params:
-                f.write("Best parameters:\n")
-                for key, value in best_params.items():
-                    f.write(f"{key}: {value}\n")
-
-            f.write("\nAll successful configurations:\n")
-            sorted_results = sorted(
-                [r for r in results if r['success']],
-                key=lambda x: x['runtime']
-            )
-            for r in sorted_results:
-                f.write(f"\nRuntime: {r['runtime']:.4f} ms\n")
-                for k, v in r['params'].items():
-                    f.write(f"{k}: {v}\n")
+        lines = [f"Tuning completed at: {stamp}", f"Best runtime: {best_runtime:.4f} ms"]
+        if best_params:
+            lines += ["Best parameters:"] + block(best_params)
+        lines += ["", "All successful configurations:"]
+        for r in sorted((r for r in results if r['success']), key=lambda r: r['runtime']):
+            lines += ["", f"Runtime: {r['runtime']:.4f} ms"] + block(r['params'])
+        (self.output_dir / 'tuning_summary.txt').write_text("\n".join(lines) + "\n")
 
 
 def main(argv=None):

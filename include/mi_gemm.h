@@ -71,6 +71,30 @@ int mi_gemm_ex(int config, int dtype, int M, int N, int K, const void* A, const 
 int mi_gemm_epilogue(int config, int dtype, int M, int N, int K, const void* A, const void* B,
                      void* C, float alpha, float beta, int c_layout, void* stream);
 
+/* ---- split-K workspace -----------------------------------------------------------------
+ * Shapes with few output tiles and a long K (decode shapes with 32 < M <= 128, 512 x 512 x
+ * 4096, ...) run as split-K: fp32 partial sums [pieces][M][N] go to a workspace and a second
+ * kernel adds them in a fixed order.  The three entry points above take that workspace from
+ * the library: one buffer per (device, stream), allocated on the first call that needs it,
+ * replaced by a larger one on demand and never freed (an enqueued launch or a captured graph
+ * may still hold its address); a stream under capture that has no large enough buffer yet
+ * runs the launch unsplit.  The reference's launchers allocate nothing per call
+ * (matmul_h100_optimal.cu:32-59); the two functions below give a caller the same property:
+ * it owns the workspace, per stream or per graph, and the library allocates nothing. */
+
+/* Bytes of workspace the library's choice of kernel wants for this call (0 when the shape
+ * does not run split-K): the largest need over the pointer alignments a launch can meet. */
+size_t mi_gemm_workspace_bytes(int config, int dtype, int M, int N, int K, int c_layout);
+
+/* mi_gemm_epilogue with a caller-owned workspace: `ws` is a device pointer, 16-byte aligned,
+ * of `ws_bytes` bytes, used only by this launch (and its successors on the same stream).
+ * Never allocates or frees.  When `ws` is NULL or smaller than the split-K choice needs, the
+ * launch runs unsplit (same tolerance, a different summation order, slower for the shapes
+ * named above).  Takes the place of the same reference launchers as mi_gemm_epilogue. */
+int mi_gemm_epilogue_ws(int config, int dtype, int M, int N, int K, const void* A, const void* B,
+                        void* C, float alpha, float beta, int c_layout, void* ws, size_t ws_bytes,
+                        void* stream);
+
 /* Plain, order-preserving GPU GEMM used as golden by the harness: one fp32 accumulator per
  * element fed in ascending k, C = (CType)(acc * alpha + beta), beta a scalar.
  * Replaces  reference_gpu_gemm(GemmParams)  (reference.h:78-90), which the reference's

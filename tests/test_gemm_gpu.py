@@ -77,14 +77,55 @@ def test_c1_square_512(mi, orc):
 
 
 def test_c2_square_8192_sampled_tiles(mi, orc):
-    tiles = orc.sample_tiles(8192, 8192, 192)
+    tiles = orc.sample_tiles(8192, 8192, 256)
     check(mi, orc, 8192, 8192, 8192, "uniform", tiles=tiles)
 
 
 @pytest.mark.parametrize("M,N,K", [(8192, 28672, 8192), (8192, 8192, 28672)])
 def test_c3_mlp_shapes_sampled_tiles(mi, orc, M, N, K):
-    tiles = orc.sample_tiles(M, N, 96)
+    tiles = orc.sample_tiles(M, N, 256)
     check(mi, orc, M, N, K, "normal", tiles=tiles)
+
+
+@pytest.mark.parametrize("M,N,K,fill", [(8192, 8192, 8192, "uniform"), (8192, 28672, 8192, "normal"),
+                                        (8192, 8192, 28672, "normal")])
+def test_c2_c3_full_matrix_against_the_gpu_golden(mi, orc, M, N, K, fill):
+    """Every element of the large benchmark shapes, the way the reference's own harness checks
+    them (matmul_h100.cu.jinja:1043-1058: whole matrix against reference_gpu_gemm): the
+    on-device golden (ascending-k fp32 sums, bit-identical to the CPU oracle, which 256
+    sampled tiles re-confirm here at full size) and the kernel's result are copied back and
+    compared element by element with the benchmark tolerance."""
+    print(f"case full matrix M={M} N={N} K={K} fill={fill}", flush=True)
+    A, B = make_inputs(orc, M, N, K, fill)
+    d = Dev(mi, A, B, M, N)
+    C = d.run(K)
+    dG = mi.DeviceBuffer(M * N * 2)
+    dG.fill_bytes(0xFF)
+    mi.reference_gpu_gemm(mi.GemmParams(M, N, K, d.dA, d.dB, dG, 1.0, 0.0))
+    mi.synchronize()
+    G = dG.to_numpy((M, N), np.uint16)
+    rep = orc.check_tolerance(C, G, K, orc.max_abs(A), orc.max_abs(B))
+    assert rep["violations"] == 0 and rep["compared"] == M * N, rep
+    tiles = orc.sample_tiles(M, N, 256)
+    ref = orc.reference_cpu_gemm(A, B, tiles=tiles)
+    for tm, tn in np.asarray(tiles).reshape(-1, 2):
+        blk = (slice(tm * 64, tm * 64 + 64), slice(tn * 64, tn * 64 + 64))
+        assert (G[blk] == ref[blk]).all(), f"golden differs from the oracle in tile ({tm}, {tn})"
+
+
+def test_c3_mlp_up_permutation_equivariance_and_determinism(mi, orc):
+    """Size-independent properties at a full MLP shape: run-to-run bit identity and
+    equivariance under row permutations of A and of B (an element's value does not depend on
+    which tile, workgroup or XCD computes it)."""
+    M, N, K = 8192, 28672, 8192
+    A, B = make_inputs(orc, M, N, K, "normal")
+    d = Dev(mi, A, B, M, N)
+    C0 = d.run(K).copy()
+    assert (d.run(K) == C0).all()
+    rng = np.random.default_rng(5)
+    pm, pn = rng.permutation(M), rng.permutation(N)
+    C1 = Dev(mi, A[pm], B[pn], M, N).run(K)
+    assert (C1 == C0[pm][:, pn]).all()
 
 
 @pytest.mark.parametrize("M", [16, 64, 128])
@@ -247,33 +288,42 @@ def test_random_shapes_and_alignments_every_tiled_kind(mi, orc):
 
 def test_non_default_streams_and_host_threads(mi, orc):
     """The ABI's stream argument: two host threads, each launching on a stream of its own
-    (created with default priority) and waiting with mi_stream_sync; shapes that use no
-    shared workspace (concurrent split-K launches are documented as the caller's to order)."""
+    (created with default priority) and waiting with mi_stream_sync.  The shapes include
+    split-K ones (decode 128 x 8192 x 8192, few tiles 384 x 512 x 4096): the library keeps one
+    workspace per stream, so the two threads' partial sums never meet."""
     import ctypes
     import threading
     hip = ctypes.CDLL("libamdhip64.so")
     L = mi._lib.load()
-    shapes = [(512, 512, 512), (1024, 768, 256), (16, 2048, 1024), (257, 515, 77), (768, 1280, 384)]
+    shapes = [(512, 512, 512), (384, 512, 4096), (16, 2048, 1024), (257, 515, 77), (128, 8192, 8192),
+              (768, 1280, 384)]
+    assert mi.workspace_bytes(384, 512, 4096) > 0 and mi.workspace_bytes(128, 8192, 8192) > 0
+    cases = []
+    for seed in range(2):
+        for M, N, K in shapes:
+            A, B = make_inputs(orc, M, N, K, "int", seed=69 + seed)
+            cases.append((seed, M, N, K, A, B, orc.reference_cpu_gemm(A, B)))
     errors = []
 
     def worker(seed):
         try:
             stream = ctypes.c_void_p()
             assert hip.hipStreamCreate(ctypes.byref(stream)) == 0
-            for rep in range(6):
-                M, N, K = shapes[(rep + seed) % len(shapes)]
-                A, B = make_inputs(orc, M, N, K, "int", seed=69 + seed)
-                ref = orc.reference_cpu_gemm(A, B)
-                dA, dB = mi.DeviceBuffer.from_numpy(A), mi.DeviceBuffer.from_numpy(B)
-                dC = mi.DeviceBuffer(M * N * 2)
-                dC.fill_bytes(0xFF)
-                mi._lib.check(L.mi_gemm_ex(-1, 0, M, N, K, dA.ptr, dB.ptr, dC.ptr, None, stream))
-                mi._lib.check(L.mi_stream_sync(stream))
-                C = dC.to_numpy((M, N), np.uint16)
-                if not (C == ref).all():
-                    errors.append(f"thread {seed} rep {rep} {M}x{N}x{K}: {int((C != ref).sum())} elements differ")
-                for b in (dA, dB, dC):
-                    b.free()
+            for rep in range(2):
+                for s, M, N, K, A, B, ref in cases:
+                    if s != seed:
+                        continue
+                    dA, dB = mi.DeviceBuffer.from_numpy(A), mi.DeviceBuffer.from_numpy(B)
+                    dC = mi.DeviceBuffer(M * N * 2)
+                    dC.fill_bytes(0xFF)
+                    for _ in range(4):      # back to back, so that the two streams' launches overlap
+                        mi._lib.check(L.mi_gemm_ex(-1, 0, M, N, K, dA.ptr, dB.ptr, dC.ptr, None, stream))
+                    mi._lib.check(L.mi_stream_sync(stream))
+                    C = dC.to_numpy((M, N), np.uint16)
+                    if not (C == ref).all():
+                        errors.append(f"thread {seed} rep {rep} {M}x{N}x{K}: {int((C != ref).sum())} elements differ")
+                    for b in (dA, dB, dC):
+                        b.free()
             assert hip.hipStreamDestroy(stream) == 0
         except Exception as e:      # surfaced in the main thread
             errors.append(f"thread {seed}: {type(e).__name__}: {e}")
@@ -286,37 +336,137 @@ def test_non_default_streams_and_host_threads(mi, orc):
     assert not errors, errors
 
 
-def test_hip_graph_replay_of_gemm_launches(mi, orc):
-    """Launches that need no workspace allocate nothing and can be captured into a HIP graph:
-    a tiled and a decode GEMM recorded on a capturing stream, replayed three times with eager
-    work and synchronisation in between, every replay compared with the eager result."""
+def test_split_k_workspace_growth_keeps_enqueued_launches_valid(mi, orc):
+    """A split-K launch that needs a larger library workspace than the stream has must not
+    free the one that launches already enqueued on that stream still use: a small split-K
+    GEMM and a large one go out back to back without a wait in between, twice, on a stream
+    that has never run split-K before."""
     import ctypes
     hip = ctypes.CDLL("libamdhip64.so")
     L = mi._lib.load()
-    cases = [(512, 512, 512), (16, 2048, 1024), (300, 200, 100)]
+    stream = ctypes.c_void_p()
+    assert hip.hipStreamCreate(ctypes.byref(stream)) == 0
+    runs = []
+    for M, N, K in [(384, 512, 4096), (128, 8192, 8192), (256, 8192, 8192)]:
+        assert mi.workspace_bytes(M, N, K) > 0
+        A, B = make_inputs(orc, M, N, K, "int")
+        runs.append((Dev(mi, A, B, M, N), M, N, K, orc.reference_cpu_gemm(A, B)))
+    need = [mi.workspace_bytes(M, N, K) for _, M, N, K, _ in runs]
+    assert need[0] < need[1] < need[2], need             # each launch outgrows the buffer before it
+    for rep in range(2):
+        for d, M, N, K, ref in runs:
+            mi._lib.check(L.mi_gemm_ex(-1, 0, M, N, K, d.dA.ptr, d.dB.ptr, d.dC.ptr, None, stream))
+        mi._lib.check(L.mi_stream_sync(stream))
+        for d, M, N, K, ref in runs:
+            C = d.dC.to_numpy((M, N), np.uint16)
+            assert (C == ref).all(), f"rep {rep} {M}x{N}x{K}: {int((C != ref).sum())} elements differ"
+            d.dC.fill_bytes(0xFF)
+    assert hip.hipStreamDestroy(stream) == 0
+
+
+def test_caller_workspace_launches_on_two_streams(mi, orc):
+    """mi_gemm_epilogue_ws: split-K partial sums in buffers the caller owns, one per stream;
+    interleaved launches on two streams, bit-exact on the integer fill and bit-identical to
+    the library-workspace entry point; a NULL or short workspace runs the launch unsplit (same
+    integers), a misaligned one is refused."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    L = mi._lib.load()
+    streams = [ctypes.c_void_p(), ctypes.c_void_p()]
+    for s in streams:
+        assert hip.hipStreamCreate(ctypes.byref(s)) == 0
+    shapes = [(128, 8192, 8192), (384, 512, 4096), (64, 4096, 8192), (512, 512, 512)]
+    per_stream = []
+    for i, s in enumerate(streams):
+        runs = []
+        for M, N, K in shapes:
+            A, B = make_inputs(orc, M, N, K, "int", seed=69 + i)
+            need = mi.workspace_bytes(M, N, K)
+            assert (need > 0) == ((M, N, K) != (512, 512, 512)), (M, N, K, need)
+            ws = mi.DeviceBuffer(max(need, 16))
+            ws.fill_bytes(0xFF)                          # NaN partials: every one must be overwritten
+            runs.append((Dev(mi, A, B, M, N), M, N, K, orc.reference_cpu_gemm(A, B), ws, need))
+        per_stream.append(runs)
+    for rep in range(3):
+        for k in range(len(shapes)):
+            for i, s in enumerate(streams):
+                d, M, N, K, ref, ws, need = per_stream[i][k]
+                mi._lib.check(L.mi_gemm_epilogue_ws(-1, 0, M, N, K, d.dA.ptr, d.dB.ptr, d.dC.ptr, 1.0, 0.0, 0,
+                                                    ws.ptr, need, s))
+    for i, s in enumerate(streams):
+        mi._lib.check(L.mi_stream_sync(s))
+        for d, M, N, K, ref, ws, need in per_stream[i]:
+            C = d.dC.to_numpy((M, N), np.uint16)
+            assert (C == ref).all(), f"stream {i} {M}x{N}x{K}: {int((C != ref).sum())} elements differ"
+    # against the library-workspace entry point on random data (same kernel, same order of sums)
+    M, N, K = 128, 8192, 8192
+    A, B = make_inputs(orc, M, N, K, "normal")
+    d = Dev(mi, A, B, M, N)
+    want = d.run(K).copy()
+    ws = mi.DeviceBuffer(mi.workspace_bytes(M, N, K))
+    for ws_ptr, ws_bytes, same in [(ws.ptr, ws.nbytes, True), (None, 0, False), (ws.ptr, 4096, False)]:
+        d.dC.fill_bytes(0xFF)
+        mi._lib.check(L.mi_gemm_epilogue_ws(-1, 0, M, N, K, d.dA.ptr, d.dB.ptr, d.dC.ptr, 1.0, 0.0, 0,
+                                            ws_ptr, ws_bytes, streams[0]))
+        mi._lib.check(L.mi_stream_sync(streams[0]))
+        C = d.dC.to_numpy((M, N), np.uint16)
+        if same:
+            assert (C == want).all()
+        else:           # unsplit: another order of sums, inside the tolerance
+            ref = orc.reference_cpu_gemm(A, B)
+            rep = orc.check_tolerance(C, ref, K, orc.max_abs(A), orc.max_abs(B))
+            assert rep["violations"] == 0, rep
+    assert L.mi_gemm_epilogue_ws(-1, 0, M, N, K, d.dA.ptr, d.dB.ptr, d.dC.ptr, 1.0, 0.0, 0, ws.ptr + 4, 1 << 20,
+                                 None) == mi._lib.MI_ERR_INVALID
+    for s in streams:
+        assert hip.hipStreamDestroy(s) == 0
+
+
+def test_hip_graph_replay_of_gemm_launches(mi, orc):
+    """A launch is kernel launches only and can be captured into a HIP graph: a tiled, a decode
+    and two split-K GEMMs (caller workspaces) recorded on a capturing stream, plus one split-K
+    shape through the library-workspace entry point on a stream that has no buffer yet (the
+    library must not allocate under capture: it records the unsplit launch).  Replayed three
+    times with eager work and synchronisation in between, every replay compared."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    L = mi._lib.load()
+    cases = [(512, 512, 512), (16, 2048, 1024), (300, 200, 100), (384, 512, 4096), (96, 4096, 8192)]
     bufs, want = [], []
     for M, N, K in cases:
         A, B = make_inputs(orc, M, N, K, "int")
         d = Dev(mi, A, B, M, N)
         want.append(d.run(K).copy())                       # eager result (also loads the kernels)
         assert (want[-1] == orc.reference_cpu_gemm(A, B)).all()
-        bufs.append((d, M, N, K))
+        ws = mi.DeviceBuffer(max(mi.workspace_bytes(M, N, K), 16))
+        bufs.append((d, M, N, K, ws))
+    assert sum(mi.workspace_bytes(M, N, K) > 0 for M, N, K in cases) >= 2
+    M2, N2, K2 = 320, 512, 4096                             # split-K shape, library workspace, fresh stream
+    assert mi.workspace_bytes(M2, N2, K2) > 0
+    A2, B2 = make_inputs(orc, M2, N2, K2, "int")
+    d2 = Dev(mi, A2, B2, M2, N2)
+    want2 = orc.reference_cpu_gemm(A2, B2)
     stream, graph, gexec = ctypes.c_void_p(), ctypes.c_void_p(), ctypes.c_void_p()
     assert hip.hipStreamCreate(ctypes.byref(stream)) == 0
     assert hip.hipStreamBeginCapture(stream, 0) == 0       # hipStreamCaptureModeGlobal
-    rcs = [L.mi_gemm_ex(-1, 0, M, N, K, d.dA.ptr, d.dB.ptr, d.dC.ptr, None, stream) for d, M, N, K in bufs]
+    rcs = [L.mi_gemm_epilogue_ws(-1, 0, M, N, K, d.dA.ptr, d.dB.ptr, d.dC.ptr, 1.0, 0.0, 0, ws.ptr, ws.nbytes, stream)
+           for d, M, N, K, ws in bufs]
+    rcs.append(L.mi_gemm_ex(-1, 0, M2, N2, K2, d2.dA.ptr, d2.dB.ptr, d2.dC.ptr, None, stream))
     assert hip.hipStreamEndCapture(stream, ctypes.byref(graph)) == 0
-    assert rcs == [0] * len(cases), rcs
+    assert rcs == [0] * (len(cases) + 1), (rcs, L.mi_last_error())
     assert hip.hipGraphInstantiate(ctypes.byref(gexec), graph, None, None, ctypes.c_size_t(0)) == 0
     for replay in range(3):
-        for d, M, N, K in bufs:
+        for d, M, N, K, ws in bufs:
             d.dC.fill_bytes(0xFF)                          # eager work between the replays
+            ws.fill_bytes(0xFF)
+        d2.dC.fill_bytes(0xFF)
         mi.synchronize()
         assert hip.hipGraphLaunch(gexec, stream) == 0
         mi._lib.check(L.mi_stream_sync(stream))
-        for (d, M, N, K), ref in zip(bufs, want):
+        for (d, M, N, K, ws), ref in zip(bufs, want):
             C = d.dC.to_numpy((M, N), np.uint16)
             assert (C == ref).all(), f"replay {replay} {M}x{N}x{K}: {int((C != ref).sum())} elements differ"
+        assert (d2.dC.to_numpy((M2, N2), np.uint16) == want2).all(), f"replay {replay} {M2}x{N2}x{K2}"
     assert hip.hipGraphExecDestroy(gexec) == 0
     assert hip.hipGraphDestroy(graph) == 0
     assert hip.hipStreamDestroy(stream) == 0
@@ -512,6 +662,49 @@ def test_harness_programs(mi):
     assert r.returncode == 0, r.stdout + r.stderr
     assert "KERNEL 1" in r.stdout
     assert re.search(r"Average elapsed time: \(\s*[\d.]+\) s, performance: \(\s*[\d.]+\) TFLOPS\. size: \(1024\)\.", r.stdout)
+
+
+def test_tuner_rendered_programs_run_and_feed_the_tuner(mi, tmp_path):
+    """The tuner's own flow on the GPU (gemm_tuner.py:34-72 of the reference: render -> compile
+    -> run `./test M m N n K k` -> parse the latency line).  The two sample configurations the
+    build rendered from template/matmul_mi355x.hip.jinja (a 16x16x32 kernel with the drain
+    barrier and a 32x32x16 two-per-CU kernel) instantiate their kernels directly, without the
+    library's dispatch.  Each runs an aligned and two ragged shapes against the on-device
+    golden; then GemmTuner.tune(prebuilt=True) sweeps them and its outputs are checked."""
+    import json
+    from h100_gemm_amd import build as lib_build
+    from h100_gemm_amd.gemm_tuner import DEFAULT_TEMPLATE, GemmTuner, LATENCY_RE
+    bindir = lib_build.TUNER_SAMPLES / "bin"
+    tuner = GemmTuner(str(DEFAULT_TEMPLATE), str(tmp_path / "out"), bin_dir=str(bindir),
+                      only=lib_build.TUNER_SAMPLE_CONFIGS, bench_args=("M", "1024", "N", "768", "K", "512", "iters", "20"))
+    names = [tuner.config_name(p) for p in tuner.configurations()]
+    assert len(names) == 2
+    for name in names:
+        exe = bindir / name
+        assert exe.exists(), f"{exe} is not built (python -m h100_gemm_amd.build)"
+        for shape in (("512", "512", "512"), ("257", "515", "77"), ("1000", "300", "1032")):
+            for extra in ([], ["dtype", "fp16"], ["fill", "uniform"]):
+                print(f"case tuner program {name} M N K = {shape} {extra}", flush=True)
+                r = subprocess.run([str(exe), "M", shape[0], "N", shape[1], "K", shape[2], "iters", "3", *extra],
+                                   capture_output=True, text=True, timeout=120)
+                assert r.returncode == 0, r.stdout + r.stderr
+                assert f"Shape M={shape[0]}, N={shape[1]}, K={shape[2]}" in r.stdout and "Correct!" in r.stdout
+                assert LATENCY_RE.search(r.stdout) and name in r.stdout, r.stdout
+    best_params, best_runtime, results = tuner.tune(prebuilt=True)
+    assert len(results) == 2 and all(r["success"] and 0 < r["runtime"] < 5 for r in results), results
+    assert best_params in lib_build.TUNER_SAMPLE_CONFIGS and best_runtime == min(r["runtime"] for r in results)
+    doc = json.loads(sorted((tmp_path / "out").glob("tuning_results_*.json"))[-1].read_text())
+    assert set(doc) == {"results", "best_params", "best_runtime", "timestamp"}
+    assert set(doc["results"][0]) == {"params", "runtime", "success", "timestamp"}
+    assert doc["best_params"] == best_params
+    assert f"Best runtime: {best_runtime:.4f} ms" in (tmp_path / "out" / "tuning_summary.txt").read_text()
+    assert f"GROUPM = {best_params['GROUP']};" in (tmp_path / "out" / "best_matmul_mi355x.hip").read_text()
+    # a configuration that was not compiled scores as a failure and the sweep goes on
+    tuner2 = GemmTuner(str(DEFAULT_TEMPLATE), str(tmp_path / "out2"), bin_dir=str(bindir),
+                       only=[dict(lib_build.TUNER_SAMPLE_CONFIGS[0], GROUP=8)] + lib_build.TUNER_SAMPLE_CONFIGS[1:],
+                       bench_args=("M", "512", "N", "512", "K", "512", "iters", "5"))
+    bp, br, res = tuner2.tune(prebuilt=True)
+    assert [r["success"] for r in res] == [False, True] and bp == lib_build.TUNER_SAMPLE_CONFIGS[1]
 
 
 def test_mfma_ceiling_program(mi):
