@@ -102,7 +102,7 @@ int choose_tile_splits(const mi::KernelEntry& e, int M, int N, int K, bool split
 }
 
 // ---- where the split-K kernels put their fp32 partial sums ----------------------------
-// Two sources, chosen by the entry point:
+// Three sources, chosen by the entry point:
 //  * LIBRARY (mi_gemm_bf16 / _ex / _epilogue): one buffer per (device, stream), allocated on
 //    first use and replaced by a larger one on demand.  A buffer is never freed while the
 //    process lives: launches already enqueued and captured graphs keep its address, so a
@@ -113,11 +113,15 @@ int choose_tile_splits(const mi::KernelEntry& e, int M, int N, int K, bool split
 //    large enough yet, the launch runs unsplit instead.
 //  * CALLER (mi_gemm_epilogue_ws): the caller's buffer, nothing is allocated; too small (or
 //    NULL) means the launch runs unsplit.
+//  * STATIC (mi_gemm_bf16_noalloc): the file-scope device array below, one copy per GPU the
+//    library runs on, of a fixed size; a shape whose partials do not fit is refused.
 // The kernels overwrite every partial they later read ([piece][M][N], all of it), so no
 // buffer needs clearing between calls.
 constexpr int kMaxDevices = 64;
+constexpr size_t kScratchBytes = MI_GEMM_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
-enum WsMode { WS_LIBRARY, WS_CALLER };
+enum WsMode { WS_LIBRARY, WS_CALLER, WS_STATIC };
 struct WsSource {
     WsMode mode = WS_LIBRARY;
     void* ptr = nullptr;      // WS_CALLER: the caller's buffer
@@ -131,6 +135,7 @@ struct StreamWs {
 struct DeviceState {
     std::vector<StreamWs> ws;        // live buffers, one per stream that ran a split-K launch
     std::vector<void*> retired;      // replaced buffers: kept until the process ends
+    unsigned char* scratch = nullptr;   // device address of `scratch` on this device
     int cus = 0;
 };
 std::mutex g_ws_mutex;
@@ -142,6 +147,22 @@ DeviceState& device_state() {
     return g_dev[dev];
 }
 
+// Device address of the static scratch array on the current device.  In host code the
+// array's name is only a handle for the runtime: the address a kernel can use comes from
+// hipGetSymbolAddress, once per device (each GPU holds its own copy at its own address).
+hipError_t static_scratch(unsigned char** out) {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    DeviceState& st = device_state();
+    if (!st.scratch) {
+        void* p = nullptr;
+        hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        st.scratch = (unsigned char*)p;
+    }
+    *out = st.scratch;
+    return hipSuccess;
+}
+
 // 0: *out holds `bytes` of workspace; 1: none to be had without allocating where that is not
 // possible (the caller runs the launch unsplit); < 0: MI_ERR_* with the message set.
 int acquire_workspace(const WsSource& src, size_t bytes, hipStream_t stream, float** out) {
@@ -149,6 +170,18 @@ int acquire_workspace(const WsSource& src, size_t bytes, hipStream_t stream, flo
     if (src.mode == WS_CALLER) {
         if (!src.ptr || src.bytes < bytes) return 1;
         *out = (float*)src.ptr;
+        return 0;
+    }
+    if (src.mode == WS_STATIC) {
+        if (bytes > kScratchBytes)
+            return fail(MI_ERR_UNSUPPORTED,
+                        "this shape's split-K partial sums need %zu bytes, the static scratch array holds %zu",
+                        bytes, kScratchBytes);
+        unsigned char* p = nullptr;
+        hipError_t e = static_scratch(&p);
+        if (e != hipSuccess)
+            return fail(MI_ERR_HIP, "hipGetSymbolAddress(scratch) failed: %s", hipGetErrorString(e));
+        *out = (float*)p;
         return 0;
     }
     std::lock_guard<std::mutex> lock(g_ws_mutex);
@@ -534,6 +567,12 @@ int mi_gemm_epilogue_ws(int config, int dtype, int M, int N, int K, const void* 
     if (c_layout == MI_C_COL_MAJOR)
         return run_gemm(config, dtype, N, M, K, B, A, C, nullptr, alpha, beta, stream, src);
     return run_gemm(config, dtype, M, N, K, A, B, C, nullptr, alpha, beta, stream, src);
+}
+
+int mi_gemm_bf16_noalloc(int M, int N, int K, const uint16_t* A, const uint16_t* B, uint16_t* C, void* stream) {
+    WsSource src;
+    src.mode = WS_STATIC;
+    return run_gemm(MI_CONFIG_AUTO, MI_DTYPE_BF16, M, N, K, A, B, C, nullptr, 1.0f, 0.0f, stream, src);
 }
 
 int mi_reference_gpu_gemm(int dtype, int M, int N, int K, const void* A, const void* B, void* C,

@@ -95,6 +95,21 @@ int mi_gemm_epilogue_ws(int config, int dtype, int M, int N, int K, const void* 
                         void* C, float alpha, float beta, int c_layout, void* ws, size_t ws_bytes,
                         void* stream);
 
+/* mi_gemm_bf16 for callers that cannot allocate device memory at all and have no workspace
+ * to pass (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  No counterpart in the reference.  Split-K partial sums go to a file-scope
+ * device array inside the library, MI_GEMM_NOALLOC_SCRATCH_BYTES per GPU, held from the
+ * moment the library is loaded until the process ends; the call makes no hipMalloc, hipFree
+ * or other allocating call.  A shape whose partial sums do not fit (pieces x M x N floats,
+ * see mi_gemm_workspace_bytes) is refused with MI_ERR_UNSUPPORTED.  Every call on a GPU
+ * shares that GPU's array: calls that run split-K and overlap on one GPU (two streams, or a
+ * graph replay next to eager calls) race on it -- keep them on one stream.  Nothing in the
+ * array needs clearing between calls: the kernels write every partial sum they later read.
+ * Results are bit-identical to mi_gemm_bf16 for the same arguments. */
+#define MI_GEMM_NOALLOC_SCRATCH_BYTES ((size_t)32 << 20)
+int mi_gemm_bf16_noalloc(int M, int N, int K, const uint16_t* A, const uint16_t* B, uint16_t* C,
+                         void* stream);
+
 /* Plain, order-preserving GPU GEMM used as golden by the harness: one fp32 accumulator per
  * element fed in ascending k, C = (CType)(acc * alpha + beta), beta a scalar.
  * Replaces  reference_gpu_gemm(GemmParams)  (reference.h:78-90), which the reference's
