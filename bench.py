@@ -52,8 +52,8 @@ MEASURED_TRAFFIC_BYTES = {
     "skinny16": (66589.6 * 2.0 + 256) * 1024,         # 0.137 GB: B is read exactly once
     "unaligned": (130105 * 2.0 + 49737) * 1024,       # 0.317 GB against 0.113 GB algorithmic
     "mlp_down": (2.7535e6 * 2.0 + 131072) * 1024,      # 5.8 GB against 1.07 GB algorithmic
-    "skinny64": ((72064 + 3086) * 2.0 + 6144 + 1024) * 1024,     # main + reduce kernels
-    "skinny128": ((80712 + 6158) * 2.0 + 12288 + 2048) * 1024,   # main + reduce kernels
+    "skinny64": ((69689 + 4114) * 2.0 + 8192 + 1024) * 1024,     # main + reduce kernels
+    "skinny128": ((73797 + 8210) * 2.0 + 16384 + 2048) * 1024,   # main + reduce kernels
 }
 
 

@@ -37,11 +37,10 @@ def _write_if_changed(path: Path, text: str) -> None:
         path.write_text(text)
 
 
-def _decode_ladder(named) -> list[tuple[int, int, str]]:
-    """(max M, config index, condition on N and K) steps of the automatic choice for decode shapes."""
+def _decode_indices(named) -> dict:
+    """role -> config index (or None) of the kernels the automatic choice for decode shapes names."""
     names = [c["name"] for c in named]
-    ladder = getattr(kc, "DECODE_LADDER", [])
-    return [(m, names.index(n), cond) for m, n, cond in ladder if n in names]
+    return {role: (names.index(n) if n in names else None) for role, n in kc.DECODE_KERNELS.items()}
 
 
 def render_sources(configs=None) -> list[Path]:
@@ -61,7 +60,7 @@ def render_sources(configs=None) -> list[Path]:
                                      tuned=[(m, n, k, [c["name"] for c in named].index(nm))
                                             for (m, n, k), nm in sorted(getattr(kc, "TUNED_SHAPES", {}).items())
                                             if nm in [c["name"] for c in named]],
-                                     skinny_index=_decode_ladder(named)))
+                                     decode_idx=_decode_indices(named)))
     # drop units of configs that no longer exist
     keep = {p.name for p in units}
     for old in GEN.glob("unit_*.hip"):
@@ -74,8 +73,8 @@ def render_sources(configs=None) -> list[Path]:
 def _stamp(src: Path) -> str:
     h = hashlib.sha1()
     for dep in [src, CSRC / "gemm_kernel.hpp", CSRC / "gemm_launch.hpp", CSRC / "gemm_ring_kernel.hpp",
-                CSRC / "gemm_skinny_kernel.hpp", CSRC / "gemm_mfma16_kernel.hpp",
-                CSRC / "gemm_stream_kernel.hpp", GEN / "kernel_table.hpp",
+                CSRC / "splitk_common.hpp", CSRC / "gemm_mfma16_kernel.hpp",
+                CSRC / "gemm_stream_kernel.hpp", CSRC / "gemm_decode_kernel.hpp", GEN / "kernel_table.hpp",
                 PKG.parent / "include" / "mi_gemm.h"]:
         h.update(dep.read_bytes())
     h.update(" ".join(HIPFLAGS).encode())

@@ -28,7 +28,7 @@
 #include <stdint.h>
 
 #include "gemm_kernel.hpp"
-#include "gemm_skinny_kernel.hpp"
+#include "splitk_common.hpp"
 
 namespace mi {
 
@@ -49,7 +49,7 @@ struct StreamConfig {
 };
 
 template <class Cfg>
-__global__ void __launch_bounds__(256) gemm_stream_kernel(const SkinnyArgs p) {
+__global__ void __launch_bounds__(256) gemm_stream_kernel(const DecodeArgs p) {
     constexpr int BM = Cfg::BM, NS = Cfg::NS, DT = Cfg::DT;
     constexpr int L = Cfg::L, STAGE = Cfg::STAGE, RING = Cfg::RING, MI = Cfg::MI;
 
@@ -182,7 +182,7 @@ __global__ void __launch_bounds__(256) gemm_stream_kernel(const SkinnyArgs p) {
 }
 
 template <class Cfg>
-hipError_t launch_stream_kernel(const SkinnyArgs& a, hipStream_t stream) {
+hipError_t launch_stream_kernel(const DecodeArgs& a, hipStream_t stream) {
     hipLaunchKernelGGL((gemm_stream_kernel<Cfg>), dim3((a.N + 31) / 32), dim3(256), 0, stream, a);
     return hipGetLastError();
 }

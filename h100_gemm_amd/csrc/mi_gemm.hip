@@ -18,7 +18,7 @@
 
 #include "../../include/mi_gemm.h"
 #include "gemm_kernel.hpp"
-#include "gemm_skinny_kernel.hpp"   // splitk_reduce_kernel
+#include "splitk_common.hpp"   // splitk_reduce_kernel
 #include "kernel_table.hpp"
 
 namespace mi {
@@ -56,22 +56,23 @@ bool shape_is_streamable(int M, int N, int K, const void* A, const void* B, cons
            (((uintptr_t)C & 7u) == 0);
 }
 
-// Split-K geometry for a decode launch.  These kernels are bound by memory latency, not by
-// CU count: about three quarters of the workgroups the chip can hold at once measured best
-// (8192 x 8192 weights, M = 64 and 128: 3 splits 30 / 38 us, 4 splits 35 / 41 us, 8 splits
-// 39 / 46 us).  The 256-row kernel (one workgroup per CU, a single slab in flight) wants
-// every CU busy instead: M = 256, 2 / 3 / 4 / 6 splits run in 87 / 67 / 62 / 77 us.
-// At least four K slabs per split.  MI_GEMM_SPLITK=<n> overrides (tuning aid).
-int choose_splits(int tiles_n, int K, int cus, int lds_bytes, int bm) {
+// Split-K geometry for a decode launch.  The decode kernel is bound by what one CU can pull
+// from HBM (~26 GB/s, whatever it keeps in flight), so it wants a workgroup on every CU: as
+// many pieces as fit into one round of the chip (128 x 8192 x 8192: 2 / 3 / 4 pieces 53 / 39.6 /
+// 35.5 us), each at least four 64-deep slabs.  Pieces are contiguous ranges of whole slabs;
+// the count is re-derived from the rounded-up piece length so that no piece is empty.
+// MI_GEMM_SPLITK=<n> overrides (tuning aid).
+int choose_splits(int tiles_n, int K, int cus) {
     static const int env = [] { const char* s = getenv("MI_GEMM_SPLITK"); return s ? atoi(s) : 0; }();
     const int slabs = K / 64;
-    const int resident = cus * (lds_bytes > 0 && 160 * 1024 / lds_bytes > 1 ? 160 * 1024 / lds_bytes : 1);
-    int splits = env > 0 ? env : bm > 128 ? cus / tiles_n : (3 * resident + 2 * tiles_n) / (4 * tiles_n);
+    int splits = env > 0 ? env : cus / tiles_n;
     if (splits > slabs / 4) splits = slabs / 4;
     if (splits < 1) splits = 1;
     if (splits > 64) splits = 64;
-    return splits;
+    const int per = (slabs + splits - 1) / splits;
+    return (slabs + per - 1) / per;
 }
+bool is_split_k_decode(int kind) { return kind == mi::KIND_DECODE; }
 
 // Split-K for the tiled 16x16x32 kernel: when a shape has so few tiles that most CUs would
 // idle (small M x N, long K), the K range is cut into pieces of whole 128-deep steps, one
@@ -291,7 +292,7 @@ int tuned_config(int M, int N, int K, bool streamable) {
     for (const TunedEntry& t : tuned_entries()) {
         if (t.M != M || t.N != N || t.K != K) continue;
         const mi::KernelEntry& e = mi::kKernels[t.config];
-        if ((e.kind == mi::KIND_SKINNY || e.kind == mi::KIND_STREAM) && (!streamable || M > e.BM)) continue;
+        if ((is_split_k_decode(e.kind) || e.kind == mi::KIND_STREAM) && (!streamable || M > e.BM)) continue;
         return t.config;
     }
     return -1;
@@ -316,9 +317,9 @@ Choice compute_choice(int requested, int M, int N, int K, bool streamable, bool 
     const mi::KernelEntry& e = mi::kKernels[c.config];
     if (e.kind == mi::KIND_MFMA16) {
         c.splits = choose_tile_splits(e, M, N, K, splittable, ptr_aligned, cus, &c.k_per_split);
-    } else if (e.kind == mi::KIND_SKINNY && streamable && M <= e.BM) {
+    } else if (is_split_k_decode(e.kind) && streamable && M <= e.BM) {
         const int tiles_n = (N + e.BN - 1) / e.BN;
-        c.splits = choose_splits(tiles_n, K, cus, e.lds_bytes, e.BM);   // <= K / 64: no empty split
+        c.splits = choose_splits(tiles_n, K, cus);   // no empty split
         c.k_per_split = ((K / 64 + c.splits - 1) / c.splits) * 64;
     }
     return c;
@@ -379,7 +380,7 @@ int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const vo
             return fail(MI_ERR_HIP, "launch of %s failed: %s", e.name, hipGetErrorString(err));
         return MI_OK;
     }
-    if (e.kind == mi::KIND_SKINNY) {
+    if (is_split_k_decode(e.kind)) {
         if (!streamable || M > e.BM)
             return fail(MI_ERR_UNSUPPORTED,
                         "config %s needs M <= %d, N %% 4 == 0, K %% 64 == 0 and 16-byte aligned operands",
@@ -465,7 +466,7 @@ int mi_gemm_config_supports(int config, int dtype, int M, int N, int K) {
     if (dtype != MI_DTYPE_BF16 && dtype != MI_DTYPE_FP16) return 0;
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     const mi::KernelEntry& e = mi::kKernels[config];
-    if (e.kind == mi::KIND_SKINNY || e.kind == mi::KIND_STREAM)
+    if (is_split_k_decode(e.kind) || e.kind == mi::KIND_STREAM)
         return M <= e.BM && N % 4 == 0 && K % 64 == 0;
     return e.launch[dtype][1] != nullptr;
 }
@@ -474,10 +475,10 @@ int mi_gemm_config_grid(int config, int M, int N, int K) {
     if (config < 0 || config >= mi::kNumKernels || M <= 0 || N <= 0 || K <= 0) return 0;
     const mi::KernelEntry& e = mi::kKernels[config];
     if (e.kind == mi::KIND_STREAM) return M > e.BM || K % 64 != 0 ? 0 : (N + e.BN - 1) / e.BN;
-    if (e.kind == mi::KIND_SKINNY) {
+    if (is_split_k_decode(e.kind)) {
         if (M > e.BM || K % 64 != 0) return 0;
         const int tiles_n = (N + e.BN - 1) / e.BN;
-        return tiles_n * choose_splits(tiles_n, K, compute_units(), e.lds_bytes, e.BM);
+        return tiles_n * choose_splits(tiles_n, K, compute_units());
     }
     const int tiles = ((M + e.BM - 1) / e.BM) * ((N + e.BN - 1) / e.BN);
     if (e.kind == mi::KIND_MFMA16) {   // split-K pieces, assuming an aligned C and no trace buffer

@@ -1,0 +1,56 @@
+// splitk_common.hpp -- what the split-K launches share: the argument block of the decode
+// kernels and the kernel that adds the fp32 partial tiles.
+//
+// A split-K launch leaves `splits` partial results [split][M][N] in an fp32 workspace;
+// splitk_reduce_kernel adds them in split order -- a fixed order, so results are reproducible
+// run to run -- applies the golden's epilogue C = (CType)(acc * alpha + beta) (reference.h:40)
+// and rounds once to the storage type.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "gemm_kernel.hpp"
+
+namespace mi {
+
+struct DecodeArgs {
+    const void* A;
+    const void* B;
+    void* C;              // storage-type output
+    float* ws;            // [splits][M][N] fp32 partials (used when splits > 1)
+    int M, N, K;
+    int lda, ldb, ldc;
+    int k_per_split;      // K range of one split (a contiguous piece), a multiple of 64
+    int splits;           // <= K / 64
+    float alpha = 1.0f;   // C = (CType)(acc * alpha + beta), applied where the sum over K is
+    float beta = 0.0f;    // complete
+};
+
+// C[m][n] = round(alpha * (sum over splits, in split order, of ws[s][m][n]) + beta); 4 elements per thread.
+template <int DT>
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restrict__ ws, void* C, int M,
+                                                            int N, int ldc, int splits, float alpha,
+                                                            float beta) {
+    const size_t idx = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    const size_t total = (size_t)M * N;
+    if (idx >= total) return;
+    float4 a = *(const float4*)(ws + idx);
+    for (int s = 1; s < splits; ++s) {
+        const float4 b = *(const float4*)(ws + (size_t)s * total + idx);
+        a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+    }
+    if (alpha != 1.0f || beta != 0.0f) {
+        a.x = mul_add_unfused(a.x, alpha, beta);
+        a.y = mul_add_unfused(a.y, alpha, beta);
+        a.z = mul_add_unfused(a.z, alpha, beta);
+        a.w = mul_add_unfused(a.w, alpha, beta);
+    }
+    const size_t m = idx / N, n = idx % N;
+    u32x2_t w;
+    w[0] = cvt_store2<DT>(a.x, a.y);
+    w[1] = cvt_store2<DT>(a.z, a.w);
+    *(u32x2_t*)((unsigned char*)C + (m * ldc + n) * 2) = w;
+}
+
+}  // namespace mi

@@ -13,8 +13,9 @@ template takes (matmul_h100.cu.jinja:9-14) -- re-cast for CDNA4:
     KIND     "tile" (two-stage kernel above), "ring" (NS-deep LDS ring, K step 32, aligned
              shapes; ragged shapes take the predicated tile kernel of the same tile),
              "mfma16" / "ring16" (the same two pipelines on the 16x16x32 MFMA with eight
-             or four waves, csrc/gemm_mfma16_kernel.hpp), or "skinny" (split-K streaming kernel for
-             M <= BM, decode shapes)
+             or four waves, csrc/gemm_mfma16_kernel.hpp), "decode" (split-K kernel for decode
+             shapes, M <= BM, whose LDS ring holds B only, csrc/gemm_decode_kernel.hpp) or
+             "stream" (single-pass decode kernel, csrc/gemm_stream_kernel.hpp)
     EPI      1: C tile transposed through LDS and written 16 bytes per lane, 0: 8-byte stores
     DRAIN    (mfma16, optional) d > 0: a second barrier early in each K step (4*d MFMAs after the
              fragment reads) frees the current LDS stage, so the next loads are spread over most
@@ -43,10 +44,10 @@ def config_name(c: dict) -> str:
         return name
     if c["KIND"] == "ring16":
         return f"q{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_n{c['NS']}_g{c['GROUP']}"
-    if c["KIND"] == "skinny":
-        return f"k{c['BM']}x{c['BN']}_n{c['NS']}"
     if c["KIND"] == "stream":
         return f"s{c['BM']}x{c['BN']}_n{c['NS']}"
+    if c["KIND"] == "decode":
+        return f"d{c['BM']}x{c['BN']}_n{c['NS']}"
     name = (f"t{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_s{c['SWZ']}_g{c['GROUP']}"
             f"_o{c['OCC']}_d{c['DTL']}_e{c['EPI']}")
     if (c.get("EWM", c["WM"]), c.get("EWN", c["WN"])) != (c["WM"], c["WN"]):
@@ -55,16 +56,16 @@ def config_name(c: dict) -> str:
 
 
 def threads(c: dict) -> int:
-    return 256 if c["KIND"] in ("skinny", "stream") else c["WM"] * c["WN"] * 64
+    return 256 if c["KIND"] in ("stream", "decode") else c["WM"] * c["WN"] * 64
 
 
 def lds_bytes(c: dict) -> int:
     if c["KIND"] in ("ring", "ring16"):
         return c["NS"] * (c["BM"] + c["BN"]) * 64
-    if c["KIND"] == "skinny":
-        return c["NS"] * (c["BM"] + c["BN"]) * 128
     if c["KIND"] == "stream":
         return 4 * c["NS"] * (c["BM"] + c["BN"]) * 128
+    if c["KIND"] == "decode":
+        return c["NS"] * c["BN"] * 128
     return 2 * (c["BM"] + c["BN"]) * 128
 
 
@@ -86,10 +87,11 @@ def is_valid_config(c: dict) -> bool:
                 and (c["NS"] - 1) * ((c["BM"] + c["BN"]) // 8) <= 63
                 and c["NS"] * (c["BM"] + c["BN"]) * 128 >= max(c["BM"], 32) * 128
                 and lds_bytes(c) <= 160 * 1024)
-    if c["KIND"] == "skinny":
-        return (c["BM"] % 32 == 0 and c["BN"] % 128 == 0 and c["NS"] >= 3
-                and ((c["BM"] + c["BN"]) // 8) % 4 == 0
-                and (c["NS"] - 1) * ((c["BM"] + c["BN"]) // 32) <= 63
+    if c["KIND"] == "decode":
+        # B-only LDS ring, A fragments in a register ring: per wave and slab BN/32 direct-to-LDS
+        # loads and BM/32 fragment loads, NS-1 slabs of them outstanding (6-bit vmcnt)
+        return (c["BM"] in (64, 128) and c["BN"] % 32 == 0 and c["NS"] >= 3
+                and (c["NS"] - 1) * (c["BM"] // 32 + c["BN"] // 32) <= 63
                 and lds_bytes(c) <= 160 * 1024)
     nt = c["WM"] * c["WN"] * 64
     if nt > 1024 or nt < 64:
@@ -177,8 +179,8 @@ def _s(BM, NS):
     return dict(KIND="stream", BM=BM, BN=32, NS=NS)
 
 
-def _k(BM, BN=128, NS=4):
-    return dict(KIND="skinny", BM=BM, BN=BN, NS=NS)
+def _d(BM, NS, BN=128):
+    return dict(KIND="decode", BM=BM, BN=BN, NS=NS)
 
 
 CONFIGS = [
@@ -210,12 +212,11 @@ CONFIGS = [
     _s(16, 5),
     _s(32, 4),
     _s(64, 3),
-    _k(32, NS=4),
-    _k(64, NS=6),
-    _k(128, NS=5),
     _m(256, 256, 2, 2, GROUP=8, DRAIN=1),
     _m(192, 192, 2, 2, DRAIN=1, EFF=0.80, EFF_E=0.91),
     _m(192, 128, 2, 2, DRAIN=1, EFF=0.74, EFF_E=0.85),
+    _d(128, NS=3),
+    _d(64, NS=4),
 ]
 
 assert all(is_valid_config(c) for c in CONFIGS), [config_name(c) for c in CONFIGS if not is_valid_config(c)]
@@ -228,50 +229,8 @@ assert len({config_name(c) for c in CONFIGS}) == len(CONFIGS)
 TUNED_SHAPES = {(8192, 8192, 28672): "m256x256_w2x2_g8_b1"}
 assert all(n in {config_name(c) for c in CONFIGS} for n in TUNED_SHAPES.values())
 
-# Automatic choice for decode shapes (the kernels' preconditions permitting): (largest M,
-# config name, further condition on N and K as a C expression), first match wins; shapes that
-# match no step go to the tiled kernels (with split-K where the time model wants it).
-# Up to M = 32 the single-pass kernel, always (16 x 1024 x 8192: 10.6 us against 13.1 us tiled;
-# 16 x 8192 x 28672: 80 against 87).  The split-K decode kernels are ahead for wide B
-# (N = 28672: 83 against 120 us at M = 64, 113 against 122 us at M = 128) and level at
-# N = 8192 for 8192 <= K <= 16384; the tiled kernels win for narrow B (M = 128, N <= 4096:
-# 11-20 against 14-21 us; M = 64, N = 2048: 12.5 against 14.2 us) and for very long K
-# (8192 x 28672: 97 against 105 us at M = 64, 106 against 136 us at M = 128).
-# Measured with B rotated through enough copies to come from HBM (selection_check, decode mode):
-#  * vocabulary-wide B with a short K (N >= 32768, K <= 4096): the split-K kernel's 128-row
-#    workgroups beat the single-pass kernel's 32-row ones (32 x 32768 x 4096: 47.5 against
-#    54 us; 32 x 65536 x 4096: 93 against 106);
-#  * 32 < M <= 64 with a short K: the single-pass kernel, no second launch (64 x 8192 x 2048:
-#    10.1 against 12.8 us; 40 x 2048 x 4096: 9.5 against 11.4; level with split-K from K = 8192),
-#    but not for wide B (64 x 28672 x 1024: 24.8 against 14.5 us for split-K);
-#  * 64 < M <= 128, N = 8192: 128x256 tiles from K = 10240 (12288: 50-53 against 54-62 us;
-#    20480: 73-77 against 87-98), except where the row pitch is a power of two (16384: 79-82
-#    against 61-68 us: the tiled kernels' rows then start in the same few memory channels).
-#  * narrow B with a long K at M <= 32 (N < 4096: fewer 32-row workgroups than CUs, each
-#    walking all of K alone) from K = 12288: split-K spreads K over the idle CUs (21 x 1792 x
-#    12288: 16.7 against 27.3 us; 32 x 2048 x 28672: 32 against 70; at K = 8192 the single pass
-#    is still ahead, 8 x 1024 x 8192: 10.3 against 15.1);
-#  * 64 < M <= 128: the split-K decode kernel from N = 12288 (74 x 14336 x 5120: 38 against
-#    42 us; 81 x 15360 x 6848: 47 against 55).
-#  * the single-pass kernel runs N / 32 workgroups, best when they fill whole rounds of the 256
-#    CUs (N = 8192, 16384): at N = 4096, 5120, 9216, 10240, 12288, 18432 (under 80 % of the
-#    last round's CUs busy) split-K is 5-30 % ahead once B is large enough to hide its
-#    second launch (32 x 5120 x 12288: 28.5 against 35.3 us; 13 x 10240 x 16384: 63 against 70;
-#    32 x 12288 x 8192: 40 against 44; but 32 x 4096 x 4096: 14 against 10.6).
-_STREAM_ROUNDS_UNDER_80 = "((N + 31) / 32) * 5 < ((((N + 31) / 32) + 255) / 256) * 1024"
-DECODE_LADDER = [(32, "k64x128_n6", "(N >= 32768 && K <= 4096) || (N < 4096 && K >= 12288) || "
-                                    "(" + _STREAM_ROUNDS_UNDER_80 + " && (long long)N * K >= 50331648LL)"),
-                 (16, "s16x32_n5", "true"), (32, "s32x32_n4", "true"),
-                 (64, "s64x32_n3", "N <= 12288 && (K <= 4096 || (N >= 4096 && K <= 6144))"),
-                 # (also for 32 < M <= 64: 48 x 6584 x 15360 45 against 56 us, 47 x 6144 x 23552 63 against 70)
-                 (128, "m128x256_w2x2_g4_b1", "N >= 4096 && N < 12288 && K >= 10240 && K < 24576 && (K & (K - 1)) != 0"),
-                 # (narrower B with a long K: 64 x 3328 x 15808 29.4 against 32.4 us tiled, 80 x 2104 x 18432
-                 # 27.2 against 29.0, 96 x 3636 x 23552 51 against 55.5)
-                 (64, "k64x128_n6", "(N >= 4096 && K < 24576) || (N >= 2048 && N < 4096 && K >= 12288 && K < 24576)"),
-                 (128, "k128x128_n5", "N >= 2048 && N < 4096 && K >= 12288"),
-                 (128, "k128x128_n5", "N >= 12288 || (N >= 8192 && K >= 8192 && K < 24576)"),
-                 # very long K: 128x256 tiles (one row of tiles covers M, B is read once) in split-K
-                 # pieces: 97 / 106 us at M = 64 / 128 against 105 / 136 us for the decode kernels
-                 # and 115-143 us for the other tiles, between which the time model cannot tell
-                 (128, "m128x256_w2x2_g4_b1", "N >= 4096 && K >= 24576")]
-assert all(n in {config_name(c) for c in CONFIGS} for _, n, _ in DECODE_LADDER)
+# The kernels the automatic choice for decode shapes names (select_decode_kernel in
+# template/kernel_table.hpp.jinja, where the thresholds and the measurements behind them are).
+DECODE_KERNELS = {"stream16": "s16x32_n5", "stream32": "s32x32_n4", "stream64": "s64x32_n3",
+                  "decode64": "d64x128_n4", "decode128": "d128x128_n3", "tile128x256": "m128x256_w2x2_g4_b1"}
+assert all(n in {config_name(c) for c in CONFIGS} for n in DECODE_KERNELS.values())

@@ -25,7 +25,7 @@ from h100_gemm_amd import kernel_configs as kc
 def candidates(decode: bool = False) -> list[int]:
     """indices of the configurations the time model chooses from (those with a measured EFF);
     with `decode` also the decode kernels of the ladder in front of the model"""
-    return [i for i, c in enumerate(kc.CONFIGS) if c.get("EFF") or (decode and c["KIND"] in ("stream", "skinny"))]
+    return [i for i, c in enumerate(kc.CONFIGS) if c.get("EFF") or (decode and c["KIND"] in ("stream", "decode"))]
 
 
 def random_shape(rng: np.random.Generator, it: int, mode: str) -> tuple[int, int, int]:

@@ -160,7 +160,7 @@ def test_every_config_uniform_within_tolerance(mi, orc, config):
 
 # ------------------------------------------------ decode (split-K streaming) kernels ----
 
-@pytest.mark.parametrize("config", all_configs(("skinny", "stream")))
+@pytest.mark.parametrize("config", all_configs(("stream", "decode")))
 def test_decode_kernels(mi, orc, config):
     from h100_gemm_amd import kernel_configs as kc
     bm = kc.CONFIGS[config]["BM"]
@@ -765,7 +765,7 @@ def test_alpha_beta_every_tiled_config_bit_exact_on_integer_fill(mi, orc, config
         check_epilogue(mi, orc, M, N, K, "int", alpha, beta, config=config, exact=True)
 
 
-@pytest.mark.parametrize("config", all_configs(("skinny", "stream")))
+@pytest.mark.parametrize("config", all_configs(("stream", "decode")))
 def test_alpha_beta_decode_kernels(mi, orc, config):
     from h100_gemm_amd import kernel_configs as kc
     bm = kc.CONFIGS[config]["BM"]
@@ -910,7 +910,7 @@ def test_alpha_beta_are_two_roundings_not_an_fma(mi, orc, alpha, beta, acc):
 
 
 def test_automatic_choice_across_regimes_bit_exact(mi, orc):
-    """The shape -> kernel choice has many branches (decode ladder with its N / K conditions,
+    """The shape -> kernel choice has many branches (decode rules with their N / K conditions,
     tuned shapes, tile model, split-K pieces, aligned / predicated twins).  Shapes on both sides
     of each boundary, integer fill, automatic choice: every result must match the oracle's bits,
     whichever kernel ran."""
@@ -927,5 +927,5 @@ def test_automatic_choice_across_regimes_bit_exact(mi, orc):
         print(f"case M={M} N={N} K={K} -> {mi.config_name(cfg)} grid {mi.config_grid(cfg, M, N, K)}", flush=True)
         check(mi, orc, M, N, K, "int", exact=True)
     # the sweep is only worth its time if it reaches the different kernel families
-    assert {"s16x32_n5", "s32x32_n4", "s64x32_n3", "k64x128_n6", "k128x128_n5"} <= seen, seen
+    assert {"s16x32_n5", "s32x32_n4", "s64x32_n3", "d64x128_n4", "d128x128_n3"} <= seen, seen
     assert any(n.startswith("m128x256") for n in seen) and any(n.startswith("m128x128") for n in seen), seen

@@ -129,7 +129,7 @@ def test_config_table(mi):
     for i, c in enumerate(kc.CONFIGS):
         assert L.mi_gemm_config_lds_bytes(i) == kc.lds_bytes(c) <= 160 * 1024
         assert kc.is_valid_config(c)
-        if c["KIND"] in ("skinny", "stream"):
+        if c["KIND"] in ("stream", "decode"):
             # decode kernels: M <= BM, whole 64-deep K slabs, N a multiple of 4; no ragged twin
             assert L.mi_gemm_config_supports(i, 0, c["BM"], 8192, 8192) == 1
             assert L.mi_gemm_config_supports(i, 0, c["BM"] + 1, 8192, 8192) == 0
@@ -148,8 +148,8 @@ def test_config_table(mi):
         assert 0 <= mi.select_config(M, N, K) < n
         assert L.mi_gemm_trace_words(M, N, K) >= 7
     kinds = {kc.CONFIGS[mi.select_config(M, 8192, 8192)]["KIND"] for M in (16, 64, 128)}
-    assert kinds <= {"skinny", "stream"}
-    assert kc.CONFIGS[mi.select_config(16, 8192, 8200)]["KIND"] != "skinny"     # K % 64 != 0
+    assert kinds <= {"stream", "decode"}
+    assert kc.CONFIGS[mi.select_config(16, 8192, 8200)]["KIND"] not in ("stream", "decode")     # K % 64 != 0
     assert kc.CONFIGS[mi.select_config(8192, 8192, 8192)]["KIND"] in ("tile", "ring", "mfma16")
     # exact shapes with a tuned entry take it; everything else goes through the cost model
     for (M, N, K), name in kc.TUNED_SHAPES.items():
@@ -182,7 +182,8 @@ def test_config_table(mi):
     assert not kc.is_valid_config(dict(KIND="tile", BM=256, BN=256, WM=2, WN=2, SWZ=1, GROUP=8, OCC=2, DTL=0, EPI=0))
     assert not kc.is_valid_config(dict(KIND="tile", BM=96, BN=256, WM=2, WN=2, SWZ=1, GROUP=8, OCC=1, DTL=0, EPI=0))
     assert not kc.is_valid_config(dict(KIND="ring", BM=256, BN=256, WM=2, WN=2, NS=5, GROUP=8))
-    assert not kc.is_valid_config(dict(KIND="skinny", BM=48, BN=128, NS=4))
+    assert not kc.is_valid_config(dict(KIND="decode", BM=48, BN=128, NS=4))
+    assert not kc.is_valid_config(dict(KIND="decode", BM=128, BN=128, NS=9))     # vmcnt is 6 bits
 
 
 def tile_of_block(pid, nwg, tiles_m, tiles_n, group):
@@ -290,7 +291,7 @@ def test_tuned_shapes_file_overrides_the_model(mi, tmp_path):
                      "1000 1000 1000 m256x192_w2x2_g4_b3\n"
                      "512 512 512 no_such_config\n"
                      "this line does not parse\n"
-                     "4096 4096 4096 k128x128_n5            # decode kernel: M too large, ignored at use\n"
+                     "4096 4096 4096 d128x128_n3            # decode kernel: M too large, ignored at use\n"
                      "64 8192 8192 s64x32_n3\n")
     code = ("import h100_gemm_amd as mi\n"
             "L = mi._lib.load()\n"
