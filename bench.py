@@ -43,17 +43,19 @@ WORKLOADS = {
     "skinny128": (128, 8192, 8192, "normal"),
     "unaligned": (4095, 6143, 3073, "uniform"),
 }
-# HBM bytes per launch of the 8192^3 kernel measured with rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE (profiles/), scaled by the same counters on a copy kernel of known size.
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (the summaries under
+# profiles/ give the commands), scaled by the same counters on a copy kernel of known size:
 # FETCH_SIZE counts KiB and reads half of what a plain 256 MiB device copy moves (131087 for
 # 262144 KiB read), so it is scaled by 2.0; WRITE_SIZE reads the copy's writes exactly (1.0).
+# workload -> (kernel configuration the counters were read on, bytes).  A profile constant,
+# not something this run measures: reported only while the run uses that same kernel.
 MEASURED_TRAFFIC_BYTES = {
-    "square8192": (787026 * 2.0 + 131083) * 1024,     # 1.75 GB against 0.40 GB algorithmic
-    "skinny16": (66589.6 * 2.0 + 256) * 1024,         # 0.137 GB: B is read exactly once
-    "unaligned": (130105 * 2.0 + 49737) * 1024,       # 0.317 GB against 0.113 GB algorithmic
-    "mlp_down": (2.7535e6 * 2.0 + 131072) * 1024,      # 5.8 GB against 1.07 GB algorithmic
-    "skinny64": ((69689 + 4114) * 2.0 + 8192 + 1024) * 1024,     # main + reduce kernels
-    "skinny128": ((73797 + 8210) * 2.0 + 16384 + 2048) * 1024,   # main + reduce kernels
+    "square8192": ("m256x256_w2x2_g4_b3", (787026 * 2.0 + 131083) * 1024),     # 1.75 GB against 0.40 GB algorithmic
+    "skinny16": ("s16x32_n5", (66589.6 * 2.0 + 256) * 1024),         # 0.137 GB: B is read exactly once
+    "unaligned": ("m256x192_w2x2_g4_b3", (130105 * 2.0 + 49737) * 1024),       # 0.317 GB against 0.113 GB algorithmic
+    "mlp_down": ("m256x256_w2x2_g8_b1", (2.7535e6 * 2.0 + 131072) * 1024),      # 5.8 GB against 1.07 GB algorithmic
+    "skinny64": ("d64x128_n4", ((69689 + 4114) * 2.0 + 8192 + 1024) * 1024),     # main + reduce kernels
+    "skinny128": ("d128x128_n3", ((73797 + 8210) * 2.0 + 16384 + 2048) * 1024),   # main + reduce kernels
 }
 
 
@@ -94,7 +96,7 @@ def sclk_under_load(launch_batch, sync) -> float | None:
     if not os.path.exists(smi):
         return None
     # not under a profiler: the child process would inherit its tool library
-    if any(k.startswith(("ROCPROF", "ROCP_", "ROCTRACER")) for k in os.environ):
+    if _under_profiler():
         return None
     try:
         proc = subprocess.Popen([smi, "--showclocks", "--json"], stdout=subprocess.PIPE,
@@ -110,6 +112,54 @@ def sclk_under_load(launch_batch, sync) -> float | None:
         return float(m.group(1)) if m else None
     except (OSError, ValueError):
         return None
+
+
+def _under_profiler() -> bool:
+    return any(k.startswith(("ROCPROF", "ROCP_", "ROCTRACER")) for k in os.environ)
+
+
+def socket_power_under_load(launch_batch, sync, seconds: float = 0.4) -> float | None:
+    """Average socket power in watts (the driver's hwmon power1_input, microwatts) sampled on
+    the host while batches of the workload's launches are in flight.  None if no such file."""
+    import glob
+    files = glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input")
+    if not files:
+        return None
+    samples = []
+    t_end = time.perf_counter() + seconds
+    try:
+        while time.perf_counter() < t_end:
+            launch_batch()                    # asynchronous: ~30 ms of work queued
+            t_batch = time.perf_counter() + 0.02
+            while time.perf_counter() < t_batch:
+                with open(files[0]) as f:
+                    samples.append(float(f.read()) * 1e-6)
+                time.sleep(0.002)
+            sync()
+    except (OSError, ValueError):
+        return None
+    tail = samples[len(samples) // 4:]        # the first quarter: the clock is still settling
+    return sum(tail) / len(tail) if tail else None
+
+
+def mfma_ceiling_same_box(fill: str) -> float | None:
+    """TFLOP/s of a loop of nothing but v_mfma_f32_16x16x32_bf16 (the kernel's instruction, its
+    accumulator tile and operand order, no memory traffic) on operands of the workload's kind,
+    run on this box right after the timed region: what the matrix pipes sustain here under
+    the chip's power limit.  The harness program h100_gemm_amd/harness/mfma_ceiling does it;
+    None when it is not built or under a profiler (the child would inherit its tool library)."""
+    import re
+    import subprocess
+    exe = ROOT / "h100_gemm_amd" / "harness" / "mfma_ceiling"
+    if not exe.exists() or _under_profiler():
+        return None
+    try:
+        out = subprocess.run([str(exe), "400", "uniform" if fill == "uniform" else "normal"], capture_output=True,
+                             text=True, timeout=60).stdout
+    except (OSError, subprocess.SubprocessError):
+        return None
+    m = re.search(r"clock [\d.]+ GHz, (\d+) TFLOP/s", out)
+    return float(m.group(1)) if m else None
 
 
 def main() -> int:
@@ -130,6 +180,8 @@ def main() -> int:
     ap.add_argument("--check-tiles", type=int, default=64, help="64x64 tiles verified against the oracle (0 = skip)")
     ap.add_argument("--no-sclk", dest="sclk", action="store_false",
                     help="do not sample the shader clock under load after the timed region")
+    ap.add_argument("--no-ceiling", dest="ceiling", action="store_false",
+                    help="do not run the MFMA-only loop (same-box ceiling) and the power sampling after the timed region")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain device-to-device copy of 256 MiB (a kernel of known HBM "
                          "traffic, for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
@@ -201,6 +253,7 @@ def main() -> int:
         for i in range(max(1, int(30.0 / ms_per_step))):
             mi.gpu_gemm(params[i % len(params)], config=cfg)
     sclk = sclk_under_load(launch_batch, mi.synchronize) if a.sclk else None
+    watts = socket_power_under_load(launch_batch, mi.synchronize) if a.ceiling else None
 
     # correctness of what was just timed, on a sample of tiles
     violations = None
@@ -219,8 +272,15 @@ def main() -> int:
     else:
         roof = {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                 "frac": gbs / PEAK_HBM_GBS}
-    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(a.workload)
+    if not hbm_bound and a.ceiling:
+        # the same-box yardstick: a slow box (they differ by +-6 % in the clock they sustain) moves
+        # `achieved` and `ceiling_same_box` together, a kernel change moves only the first
+        ceiling = mfma_ceiling_same_box(fill)
+        roof["ceiling_same_box"] = ceiling
+        roof["frac_of_ceiling"] = tflops / ceiling if ceiling else None
     roof["kernel"] = mi.config_name(cfg)
+    traffic_kernel, traffic = MEASURED_TRAFFIC_BYTES.get(a.workload, (None, None))
+    roof["traffic"] = traffic if traffic_kernel == roof["kernel"] else None
     roof["avg_launch_us"] = ms_per_step * 1e3
 
     cpu = cpu_baseline(orc, A, B, a.cpu_tiles) if a.cpu_tiles > 0 else None
@@ -235,7 +295,8 @@ def main() -> int:
         "config": {"workload": f"{a.workload}: M={M} N={N} K={K}, A,B {fill} seeded bf16, fp32 accumulate, bf16 out",
                    "kernel_config": mi.config_name(cfg), "device": props["name"] or props["arch"],
                    "compute_units": props["compute_units"], "peak_clock_mhz": props["clock_khz"] / 1000,
-                   "sclk_mhz_under_load": sclk},
+                   "sclk_mhz_under_load": sclk, "socket_power_w_under_load": watts,
+                   "joules_per_launch": watts * ms_per_step * 1e-3 if watts else None},
         "pct_of_bf16_mfma_peak": 100.0 * tflops / PEAK_BF16_TFLOPS,
         "achieved_gbs_algorithmic": gbs,
         "tolerance_violations": violations,

@@ -18,6 +18,7 @@ from pathlib import Path
 
 from jinja2 import Template
 
+from . import isa_check
 from . import kernel_configs as kc
 
 PKG = Path(__file__).resolve().parent
@@ -75,10 +76,31 @@ def _stamp(src: Path) -> str:
     for dep in [src, CSRC / "gemm_kernel.hpp", CSRC / "gemm_launch.hpp", CSRC / "gemm_ring_kernel.hpp",
                 CSRC / "splitk_common.hpp", CSRC / "gemm_mfma16_kernel.hpp",
                 CSRC / "gemm_stream_kernel.hpp", CSRC / "gemm_decode_kernel.hpp", GEN / "kernel_table.hpp",
-                PKG.parent / "include" / "mi_gemm.h"]:
+                PKG.parent / "include" / "mi_gemm.h", PKG / "isa_check.py"]:
         h.update(dep.read_bytes())
     h.update(" ".join(HIPFLAGS).encode())
     return h.hexdigest()
+
+
+def _asm_path(obj: Path) -> Path:
+    """where `-save-temps=obj` leaves the device assembly text of a unit"""
+    return obj.with_name(obj.stem + "-hip-amdgcn-amd-amdhsa-gfx950.s")
+
+
+def _check_unit(src: Path, obj: Path) -> None:
+    """The invariants of the generated code that the inline asm relies on (isa_check): a unit
+    that breaks one fails the build."""
+    asm = _asm_path(obj)
+    if not asm.exists():
+        raise RuntimeError(f"{src.name}: no assembly text at {asm} (needed for the M0 / scratch checks)")
+    text = asm.read_text()
+    cfg = next((c for c in kc.CONFIGS if src.name == f"unit_{kc.config_name(c)}.hip"), None)
+    if cfg is None:
+        return                                  # not a kernel unit
+    # {bf16, fp16} x {aligned, predicated} x {plain, trace, split-K} for the 16x16x32 kernel
+    isa_check.check_m0(src.name, text, need_kernels=8 if cfg["KIND"] == "mfma16" else 1)
+    if cfg["KIND"] == "mfma16" and cfg.get("EFF"):
+        isa_check.check_no_scratch(src.name, text)
 
 
 def _compile(src: Path, force: bool) -> Path:
@@ -87,10 +109,15 @@ def _compile(src: Path, force: bool) -> Path:
     want = _stamp(src)
     if not force and obj.exists() and stamp.exists() and stamp.read_text() == want:
         return obj
-    cmd = [HIPCC, *HIPFLAGS, "-c", str(src), "-o", str(obj)]
+    cmd = [HIPCC, *HIPFLAGS, "-save-temps=obj", "-c", str(src), "-o", str(obj)]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src.name}:\n{r.stderr[-4000:]}")
+    # of the intermediate files only the device assembly text is kept
+    for tmp in list(obj.parent.glob(obj.stem + "-*")) + list(obj.parent.glob(src.name + "-*")):
+        if tmp != _asm_path(obj):
+            tmp.unlink()
+    _check_unit(src, obj)
     stamp.write_text(want)
     return obj
 

@@ -21,7 +21,9 @@ CDNA4:
 Additions: ``prebuild()`` compiles every valid configuration in parallel into
 ``<output_dir>/bin`` (hipcc cross-compiles without a GPU, so the slow part can run on a
 build host), ``tune(prebuilt=True)`` then only runs the binaries; ``resume_from`` reloads an
-earlier results JSON and skips what it already holds.
+earlier results JSON and skips what it already holds; ``--write-tuned FILE MxNxK ...``
+(``tune_library_choice``) times the library's compiled candidates for given shapes and writes
+the winners in the format ``MI_GEMM_TUNED_FILE`` reads.
 """
 from __future__ import annotations
 
@@ -257,6 +259,66 @@ class GemmTuner:
         (self.output_dir / 'tuning_summary.txt').write_text("\n".join(lines) + "\n")
 
 
+def tune_library_choice(shapes, out_file: Optional[str] = None, margin: float = 0.02):
+    """The run-time form of the tuner's persisted results: for every (M, N, K) time the
+    library's automatic choice and each compiled candidate of its time model on the GPU
+    (through the C ABI, best of three batches of ~30 ms of back-to-back launches) and, where a candidate
+    beats the automatic choice by more than `margin`, append `M N K config-name` to
+    `out_file` -- the format MI_GEMM_TUNED_FILE reads (keyed on all of M, N, K, where the
+    reference keys its cached descriptors on M alone, matmul_utils.cuh:49-51).
+    Returns [(shape, automatic config, its ms, best config, its ms)]."""
+    import numpy as np
+
+    import h100_gemm_amd as mi
+    lib = mi._lib.load()
+    cands = [i for i, c in enumerate(kc.CONFIGS) if c.get("EFF") or c["KIND"] in ("stream", "decode")]
+
+    def time_config(config, params, launches):
+        for i in range(max(3, launches // 4)):
+            mi.gpu_gemm(params[i % len(params)], config=config)
+        mi.synchronize()
+        best = float("inf")
+        for _ in range(3):
+            timer = mi.GPUTimer()
+            timer.tick()
+            for i in range(launches):
+                mi.gpu_gemm(params[i % len(params)], config=config)
+            timer.tick()
+            best = min(best, timer.report_last_ms() / launches)
+        return best
+
+    rng = np.random.default_rng(1)
+    block = rng.integers(0x3000, 0x3F80, size=1 << 22, dtype=np.uint16) | (rng.integers(0, 2, size=1 << 22, dtype=np.uint16) << 15)
+    out = []
+    for M, N, K in shapes:
+        A, B = np.resize(block, (M, K)), np.resize(block[::-1], (N, K))
+        # decode shapes stream their weights from HBM in real use: enough copies of B to exceed
+        # the 256 MB memory-side cache, visited in turn
+        copies = min(8, -(-(600 << 20) // B.nbytes)) if M <= 128 else 1
+        dA, dC = mi.DeviceBuffer.from_numpy(A), mi.DeviceBuffer(M * N * 2)
+        dBs = [mi.DeviceBuffer.from_numpy(B) for _ in range(copies)]
+        params = [mi.GemmParams(M, N, K, dA, dB, dC) for dB in dBs]
+        launches = int(min(200, max(10, 3e-2 / (2.0 * M * N * K / 1.2e15 + 5e-6))))
+        auto = mi.select_config(M, N, K)
+        t_auto = time_config(mi.MI_CONFIG_AUTO, params, launches)
+        times = {c: time_config(c, params, launches) for c in cands if lib.mi_gemm_config_supports(c, 0, M, N, K)}
+        t_auto = min(t_auto, time_config(mi.MI_CONFIG_AUTO, params, launches))
+        best = min(times, key=times.get)
+        print(f"{M}x{N}x{K}: automatic choice {mi.config_name(auto)} {t_auto * 1e3:.1f} us, "
+              f"best candidate {mi.config_name(best)} {times[best] * 1e3:.1f} us", flush=True)
+        if out_file and t_auto > times[best] * (1.0 + margin):
+            with open(out_file, "a") as f:
+                f.write(f"{M} {N} {K} {mi.config_name(best)}\n")
+        out.append(((M, N, K), mi.config_name(auto), t_auto, mi.config_name(best), times[best]))
+        for b in [dA, dC] + dBs:
+            b.free()
+    if out:
+        losses = [max(0.0, t_auto / t_best - 1.0) for _, _, t_auto, _, t_best in out]
+        print(f"{len(out)} shapes: the automatic choice loses {100 * sum(losses) / len(losses):.2f} % on average to the "
+              f"best candidate, more than 4 % on {sum(l > 0.04 for l in losses)}, at worst {100 * max(losses):.0f} %")
+    return out
+
+
 def main(argv=None):
     import argparse
     ap = argparse.ArgumentParser(description="MI355X GEMM tuner")
@@ -267,14 +329,22 @@ def main(argv=None):
     ap.add_argument("--shape", nargs=3, type=int, default=[5120, 5120, 4096], metavar=("M", "N", "K"))
     ap.add_argument("--fill", default=None, choices=["int", "uniform", "normal"])
     ap.add_argument("-j", "--jobs", type=int, default=8)
+    ap.add_argument("--write-tuned", metavar="FILE", default=None,
+                    help="instead of sweeping the template: time the library's compiled candidates for the shapes "
+                         "given as MxNxK arguments and append `M N K config-name` lines (MI_GEMM_TUNED_FILE format) "
+                         "where one beats the automatic choice")
+    ap.add_argument("shapes", nargs="*", help="shapes as MxNxK (with --write-tuned)")
     a = ap.parse_args(argv)
+    if a.write_tuned:
+        tune_library_choice([tuple(int(v) for v in s.split("x")) for s in a.shapes], a.write_tuned)
+        return 0
     bench_args = ["M", str(a.shape[0]), "N", str(a.shape[1]), "K", str(a.shape[2])]
     if a.fill:
         bench_args += ["fill", a.fill]
     tuner = GemmTuner(str(DEFAULT_TEMPLATE), a.output_dir, bench_args=bench_args, resume_from=a.resume)
     if a.prebuild:
         built = tuner.prebuild(a.jobs)
-        print(f"compiled {sum(built.values())} of {len(built)} configurations into {tuner.output_dir / 'bin'}")
+        print(f"compiled {sum(built.values())} of {len(built)} configurations into {tuner.bin_dir}")
         return 0 if all(built.values()) else 1
     best_params, best_runtime, results = tuner.tune(prebuilt=a.prebuilt)
 

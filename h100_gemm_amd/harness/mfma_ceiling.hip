@@ -5,7 +5,7 @@
 // power limited: the issue rate is the same for every data set (~16.3 cycles per MFMA), the
 // clock is not -- zeros run near the peak clock, random bf16 operands far below it.
 //
-//     ./mfma_ceiling [milliseconds per data set]         default 300
+//     ./mfma_ceiling [milliseconds per data set] [zeros|uniform|normal]     default 300, all three
 //
 // One line per data set: cycles per MFMA (the shader-cycle counter of one wave), shader clock
 // (cycles / wall time), and the rate of the whole chip in TFLOP/s.  No memory traffic, no
@@ -70,6 +70,7 @@ static uint16_t to_bf16(float f) {
 
 int main(int argc, char** argv) {
     const double ms_per_set = argc > 1 ? atof(argv[1]) : 300.0;
+    const char* only = argc > 2 ? argv[2] : nullptr;       // one data set: "zeros", "uniform" or "normal"
     int dev = 0, cus = 0;
     HIP_OK(hipGetDevice(&dev));
     HIP_OK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
@@ -87,6 +88,7 @@ int main(int argc, char** argv) {
     struct Set { const char* name; int kind; };
     const Set sets[] = {{"zeros", 0}, {"uniform [-1,1) bf16", 1}, {"normal(0,1) bf16", 2}};
     for (const Set& set : sets) {
+        if (only && strncmp(set.name, only, strlen(only)) != 0) continue;
         std::vector<uint16_t> h(4096 * 8);
         uint64_t x = 0x9E3779B97F4A7C15ull;
         auto next = [&]() {

@@ -267,18 +267,14 @@ int main() {
     assert (got[4096:] == orc.fill_normal((4096,), 69, 2, 0.02)).all()
 
 
-def test_selection_check_tool_is_seeded_and_knows_the_candidates():
-    """the tuning aid that times the automatic choice against its candidates: same seed, same
-    shapes; its candidate list is the model's (configurations with a measured rate)"""
-    import numpy as np
-    from h100_gemm_amd import kernel_configs as kc, selection_check as sc
-    a = [sc.random_shape(np.random.default_rng(5), i, m) for i in range(6) for m in ("general", "shortk", "midm")]
-    b = [sc.random_shape(np.random.default_rng(5), i, m) for i in range(6) for m in ("general", "shortk", "midm")]
-    assert a == b and all(m >= 1 and n >= 1 and k >= 1 and m * n * k <= 4.1e11 for m, n, k in a)
-    names = [kc.config_name(kc.CONFIGS[i]) for i in sc.candidates()]
-    assert len(names) == 7 and all(n.startswith("m") for n in names)
-    p = sc.bf16_pattern((5, 7), 1)
-    assert p.shape == (5, 7) and p.dtype == np.uint16 and ((p & 0x7FFF) < 0x3F80).all()
+def test_tuner_write_tuned_mode_without_shapes_writes_nothing(mi, tmp_path):
+    """`gemm_tuner --write-tuned FILE MxNxK ...` times the library's compiled candidates on the
+    GPU (tune_library_choice); with no shapes it touches neither the GPU nor the file"""
+    from h100_gemm_amd import gemm_tuner
+    out = tmp_path / "tuned.txt"
+    assert gemm_tuner.main(["--write-tuned", str(out)]) == 0
+    assert not out.exists()
+    assert gemm_tuner.tune_library_choice([], str(out)) == []
 
 
 def test_tuned_shapes_file_overrides_the_model(mi, tmp_path):
