@@ -37,6 +37,7 @@ WORKLOADS = {
     "square512": (512, 512, 512, "uniform"),
     "square8192": (8192, 8192, 8192, "uniform"),
     "mlp_up": (8192, 28672, 8192, "normal"),
+    "mlp_up": ("m256x256_w2x2_g4_b3", (2753408 * 2.0 + 458779) * 1024),         # 6.1 GB against 1.34 GB algorithmic
     "mlp_down": (8192, 8192, 28672, "normal"),
     "skinny16": (16, 8192, 8192, "normal"),
     "skinny64": (64, 8192, 8192, "normal"),
@@ -53,6 +54,7 @@ MEASURED_TRAFFIC_BYTES = {
     "square8192": ("m256x256_w2x2_g4_b3", (787026 * 2.0 + 131083) * 1024),     # 1.75 GB against 0.40 GB algorithmic
     "skinny16": ("s16x32_n5", (66589.6 * 2.0 + 256) * 1024),         # 0.137 GB: B is read exactly once
     "unaligned": ("m256x192_w2x2_g4_b3", (130105 * 2.0 + 49737) * 1024),       # 0.317 GB against 0.113 GB algorithmic
+    "mlp_up": ("m256x256_w2x2_g4_b3", (2753408 * 2.0 + 458779) * 1024),         # 6.1 GB against 1.34 GB algorithmic
     "mlp_down": ("m256x256_w2x2_g8_b1", (2.7535e6 * 2.0 + 131072) * 1024),      # 5.8 GB against 1.07 GB algorithmic
     "skinny64": ("d64x128_n4", ((69689 + 4114) * 2.0 + 8192 + 1024) * 1024),     # main + reduce kernels
     "skinny128": ("d128x128_n3", ((73797 + 8210) * 2.0 + 16384 + 2048) * 1024),   # main + reduce kernels

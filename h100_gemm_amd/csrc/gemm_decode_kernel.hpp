@@ -297,13 +297,11 @@ gemm_decode_kernel(const DecodeArgs p) {
 template <class Cfg>
 hipError_t launch_decode_kernel(const DecodeArgs& a, hipStream_t stream) {
     dim3 grid((a.N + Cfg::BN - 1) / Cfg::BN, a.splits);
-    hipLaunchKernelGGL((gemm_decode_kernel<Cfg>), grid, dim3(256), 0, stream, a);
-    hipError_t e = hipGetLastError();
+    hipError_t e = launch_kernel(gemm_decode_kernel<Cfg>, grid, dim3(256), stream, a);
     if (e != hipSuccess || a.splits == 1) return e;
     const size_t quads = ((size_t)a.M * a.N + 3) / 4;
-    hipLaunchKernelGGL((splitk_reduce_kernel<Cfg::DT>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0,
-                       stream, a.ws, a.C, a.M, a.N, a.ldc, a.splits, a.alpha, a.beta);
-    return hipGetLastError();
+    return launch_kernel(splitk_reduce_kernel<Cfg::DT>, dim3((unsigned)((quads + 255) / 256)), dim3(256), stream,
+                         a.ws, a.C, a.M, a.N, a.ldc, a.splits, a.alpha, a.beta);
 }
 
 }  // namespace mi

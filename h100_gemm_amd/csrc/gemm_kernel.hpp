@@ -32,6 +32,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <tuple>
+#include <type_traits>
+
 #include <type_traits>
 
 namespace mi {
@@ -59,6 +62,19 @@ struct GemmArgs {
     float alpha = 1.0f;      // C = (CType)(acc * alpha + beta), beta a plain scalar added to
     float beta = 0.0f;       // every element (reference.h:40)
 };
+
+// Launch `kernel` with the given arguments and return the status of THIS launch.
+// (hipLaunchKernelGGL + hipGetLastError would also report -- and clear -- an error that some
+// earlier, unrelated call of the process left behind, as a failure of the GEMM.)
+template <class... KArgs, class... Args>
+inline hipError_t launch_kernel(void (*kernel)(KArgs...), dim3 grid, dim3 block, hipStream_t stream, Args... args) {
+    // one slot per kernel parameter, converted to the parameter's own type
+    std::tuple<std::decay_t<KArgs>...> held{static_cast<std::decay_t<KArgs>>(args)...};
+    void* ptrs[sizeof...(KArgs)];
+    int n = 0;
+    std::apply([&](auto&... a) { ((ptrs[n++] = (void*)&a), ...); }, held);
+    return hipLaunchKernel((const void*)kernel, grid, block, ptrs, 0, stream);
+}
 
 // Compile-time description of one kernel variant -- the knobs the tuner sweeps.
 //   BM x BN      macro tile of one workgroup (K step is 64 elements = one 128-byte LDS row)

@@ -12,8 +12,7 @@ namespace mi {
 template <class Cfg, bool TRACE = false>
 hipError_t launch_tile_kernel(const GemmArgs& args, hipStream_t stream) {
     const int grid = args.tiles_m * args.tiles_n;
-    hipLaunchKernelGGL((gemm_tile_kernel<Cfg, TRACE>), dim3(grid), dim3(Cfg::NT), 0, stream, args);
-    return hipGetLastError();
+    return launch_kernel(gemm_tile_kernel<Cfg, TRACE>, dim3(grid), dim3(Cfg::NT), stream, args);
 }
 
 }  // namespace mi

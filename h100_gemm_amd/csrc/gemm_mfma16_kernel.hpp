@@ -757,8 +757,7 @@ gemm_ring16_kernel(const GemmArgs p) {
 template <class Cfg, bool TRACE = false>
 hipError_t launch_ring16_kernel(const GemmArgs& args, hipStream_t stream) {
     const int grid = args.tiles_m * args.tiles_n;
-    hipLaunchKernelGGL((gemm_ring16_kernel<Cfg, TRACE>), dim3(grid), dim3(Cfg::NT), 0, stream, args);
-    return hipGetLastError();
+    return launch_kernel(gemm_ring16_kernel<Cfg, TRACE>, dim3(grid), dim3(Cfg::NT), stream, args);
 }
 
 template <class Cfg, bool TRACE = false>
@@ -766,11 +765,9 @@ hipError_t launch_mfma16_kernel(const GemmArgs& args, hipStream_t stream) {
     const int grid = args.tiles_m * args.tiles_n;
     if (args.splits > 1) {
         if constexpr (TRACE) return hipErrorInvalidValue;   // no trace records from split-K launches
-        hipLaunchKernelGGL((gemm_mfma16_kernel<Cfg, false, true>), dim3(grid, args.splits), dim3(Cfg::NT), 0, stream, args);
-    } else {
-        hipLaunchKernelGGL((gemm_mfma16_kernel<Cfg, TRACE>), dim3(grid), dim3(Cfg::NT), 0, stream, args);
+        return launch_kernel(gemm_mfma16_kernel<Cfg, false, true>, dim3(grid, args.splits), dim3(Cfg::NT), stream, args);
     }
-    return hipGetLastError();
+    return launch_kernel(gemm_mfma16_kernel<Cfg, TRACE>, dim3(grid), dim3(Cfg::NT), stream, args);
 }
 
 }  // namespace mi

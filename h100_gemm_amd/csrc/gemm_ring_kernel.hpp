@@ -266,8 +266,7 @@ gemm_ring_kernel(const GemmArgs p) {
 template <class Cfg, bool TRACE = false>
 hipError_t launch_ring_kernel(const GemmArgs& args, hipStream_t stream) {
     const int grid = args.tiles_m * args.tiles_n;
-    hipLaunchKernelGGL((gemm_ring_kernel<Cfg, TRACE>), dim3(grid), dim3(Cfg::NT), 0, stream, args);
-    return hipGetLastError();
+    return launch_kernel(gemm_ring_kernel<Cfg, TRACE>, dim3(grid), dim3(Cfg::NT), stream, args);
 }
 
 }  // namespace mi

@@ -83,6 +83,11 @@ __global__ void __launch_bounds__(256) gemm_stream_kernel(const DecodeArgs p) {
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                      :: "s"(dst), "v"(voff), "s"(rsrc) : "memory");
     };
+    // B is read once: non-temporal, so that it does not push A (re-read by every workgroup) out of the L2s
+    auto dma_nt = [&](const __amdgpu_buffer_rsrc_t& rsrc, uint32_t voff, uint32_t dst) __attribute__((always_inline)) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen nt lds"
+                     :: "s"(dst), "v"(voff), "s"(rsrc) : "memory");
+    };
     // this lane's byte offsets inside A and B for instruction q of a slab (k offset added later)
     uint32_t voff[L];
 #pragma unroll
@@ -101,9 +106,10 @@ __global__ void __launch_bounds__(256) gemm_stream_kernel(const DecodeArgs p) {
         gs += 4;
         while (gs >= KT) gs -= KT;
 #pragma unroll
-        for (int q = 0; q < L; ++q)
-            dma(live ? (q * 8 < BM ? rsrcA : rsrcB) : rsrcNone, voff[q] + kb,
-                ring_base + (uint32_t)(s * STAGE + q * 1024));
+        for (int q = 0; q < L; ++q) {
+            if (q * 8 < BM) dma(live ? rsrcA : rsrcNone, voff[q] + kb, ring_base + (uint32_t)(s * STAGE + q * 1024));
+            else dma_nt(live ? rsrcB : rsrcNone, voff[q] + kb, ring_base + (uint32_t)(s * STAGE + q * 1024));
+        }
     };
 
     // fragment reads: lane holds row (lane & 31), k chunk 2*ks + (lane >> 5).  With BM = 16
@@ -183,8 +189,7 @@ __global__ void __launch_bounds__(256) gemm_stream_kernel(const DecodeArgs p) {
 
 template <class Cfg>
 hipError_t launch_stream_kernel(const DecodeArgs& a, hipStream_t stream) {
-    hipLaunchKernelGGL((gemm_stream_kernel<Cfg>), dim3((a.N + 31) / 32), dim3(256), 0, stream, a);
-    return hipGetLastError();
+    return launch_kernel(gemm_stream_kernel<Cfg>, dim3((a.N + 31) / 32), dim3(256), stream, a);
 }
 
 }  // namespace mi

@@ -423,13 +423,11 @@ int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const vo
     if (args.splits > 1) {
         const size_t quads = ((size_t)M * N + 3) / 4;
         const dim3 rgrid((unsigned)((quads + 255) / 256));
-        if (dtype == MI_DTYPE_BF16)
-            hipLaunchKernelGGL((mi::splitk_reduce_kernel<mi::DT_BF16>), rgrid, dim3(256), 0, (hipStream_t)stream,
-                               args.ws, C, M, N, N, args.splits, alpha, beta);
-        else
-            hipLaunchKernelGGL((mi::splitk_reduce_kernel<mi::DT_FP16>), rgrid, dim3(256), 0, (hipStream_t)stream,
-                               args.ws, C, M, N, N, args.splits, alpha, beta);
-        err = hipGetLastError();
+        err = dtype == MI_DTYPE_BF16
+                  ? mi::launch_kernel(mi::splitk_reduce_kernel<mi::DT_BF16>, rgrid, dim3(256), (hipStream_t)stream,
+                                      args.ws, C, M, N, N, args.splits, alpha, beta)
+                  : mi::launch_kernel(mi::splitk_reduce_kernel<mi::DT_FP16>, rgrid, dim3(256), (hipStream_t)stream,
+                                      args.ws, C, M, N, N, args.splits, alpha, beta);
         if (err != hipSuccess)
             return fail(MI_ERR_HIP, "launch of the split-K reduction failed: %s", hipGetErrorString(err));
     }

@@ -90,12 +90,13 @@ namespace mi {
 hipError_t launch_reference_gpu_gemm(int dtype, int M, int N, int K, const void* A, const void* B,
                                      void* C, float alpha, float beta, hipStream_t stream) {
     dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
-    if (dtype == MI_DTYPE_BF16)
-        hipLaunchKernelGGL(naive_gemm_kernel<MI_DTYPE_BF16>, grid, block, 0, stream, M, N, K,
-                           (const uint16_t*)A, (const uint16_t*)B, (uint16_t*)C, alpha, beta);
-    else
-        hipLaunchKernelGGL(naive_gemm_kernel<MI_DTYPE_FP16>, grid, block, 0, stream, M, N, K,
-                           (const uint16_t*)A, (const uint16_t*)B, (uint16_t*)C, alpha, beta);
-    return hipGetLastError();
+    // the status of this launch (not an error some earlier call of the process left behind)
+    const uint16_t* a = (const uint16_t*)A;
+    const uint16_t* b = (const uint16_t*)B;
+    uint16_t* c = (uint16_t*)C;
+    void* args[] = {&M, &N, &K, &a, &b, &c, &alpha, &beta};
+    const void* kernel = dtype == MI_DTYPE_BF16 ? (const void*)naive_gemm_kernel<MI_DTYPE_BF16>
+                                                : (const void*)naive_gemm_kernel<MI_DTYPE_FP16>;
+    return hipLaunchKernel(kernel, grid, block, args, 0, stream);
 }
 }  // namespace mi

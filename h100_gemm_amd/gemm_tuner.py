@@ -259,7 +259,7 @@ class GemmTuner:
         (self.output_dir / 'tuning_summary.txt').write_text("\n".join(lines) + "\n")
 
 
-def tune_library_choice(shapes, out_file: Optional[str] = None, margin: float = 0.02):
+def tune_library_choice(shapes, out_file: Optional[str] = None, margin: float = 0.02, all_times: bool = False):
     """The run-time form of the tuner's persisted results: for every (M, N, K) time the
     library's automatic choice and each compiled candidate of its time model on the GPU
     (through the C ABI, best of three batches of ~30 ms of back-to-back launches) and, where a candidate
@@ -306,6 +306,8 @@ def tune_library_choice(shapes, out_file: Optional[str] = None, margin: float = 
         best = min(times, key=times.get)
         print(f"{M}x{N}x{K}: automatic choice {mi.config_name(auto)} {t_auto * 1e3:.1f} us, "
               f"best candidate {mi.config_name(best)} {times[best] * 1e3:.1f} us", flush=True)
+        if all_times:
+            print("    " + " ".join(f"{mi.config_name(c)}={t * 1e3:.1f}" for c, t in sorted(times.items(), key=lambda ct: ct[1])), flush=True)
         if out_file and t_auto > times[best] * (1.0 + margin):
             with open(out_file, "a") as f:
                 f.write(f"{M} {N} {K} {mi.config_name(best)}\n")
@@ -333,10 +335,11 @@ def main(argv=None):
                     help="instead of sweeping the template: time the library's compiled candidates for the shapes "
                          "given as MxNxK arguments and append `M N K config-name` lines (MI_GEMM_TUNED_FILE format) "
                          "where one beats the automatic choice")
+    ap.add_argument("--all-times", action="store_true", help="with --write-tuned: print every candidate's time")
     ap.add_argument("shapes", nargs="*", help="shapes as MxNxK (with --write-tuned)")
     a = ap.parse_args(argv)
     if a.write_tuned:
-        tune_library_choice([tuple(int(v) for v in s.split("x")) for s in a.shapes], a.write_tuned)
+        tune_library_choice([tuple(int(v) for v in s.split("x")) for s in a.shapes], a.write_tuned, all_times=a.all_times)
         return 0
     bench_args = ["M", str(a.shape[0]), "N", str(a.shape[1]), "K", str(a.shape[2])]
     if a.fill:
