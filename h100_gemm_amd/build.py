@@ -73,9 +73,8 @@ def render_sources(configs=None) -> list[Path]:
 
 def _stamp(src: Path) -> str:
     h = hashlib.sha1()
-    for dep in [src, CSRC / "gemm_kernel.hpp", CSRC / "gemm_launch.hpp", CSRC / "gemm_ring_kernel.hpp",
-                CSRC / "splitk_common.hpp", CSRC / "gemm_mfma16_kernel.hpp",
-                CSRC / "gemm_stream_kernel.hpp", CSRC / "gemm_decode_kernel.hpp", GEN / "kernel_table.hpp",
+    # every header of csrc/ (a unit includes a few of them; rebuilding all on any change is cheap)
+    for dep in [src, *sorted(CSRC.glob("*.hpp")), GEN / "kernel_table.hpp",
                 PKG.parent / "include" / "mi_gemm.h", PKG / "isa_check.py"]:
         h.update(dep.read_bytes())
     h.update(" ".join(HIPFLAGS).encode())

@@ -1,0 +1,216 @@
+// gemm_wavek_kernel.hpp -- gfx950 GEMM kernel for outputs of few tiles with a long K:
+//
+//   C[M,N] = A[M,K] . B[N,K]^T     small tiles, K split over the four waves of a workgroup,
+//                                  one kernel, no workspace
+//
+// A 512 x 512 or 1024 x 1024 output has 16 or 64 tiles of 128 x 128: most of the chip idles,
+// or K is cut into pieces whose partial sums make a round trip through memory and a second
+// launch.  Here the tile is small enough (32 x 32 ... 96 x 64) for every CU to own one, and
+// what a small tile loses -- each wave of a 2 x 2 wave grid would re-read most of the tile's
+// LDS for very few MFMAs -- is avoided by splitting K instead of the tile:
+//   * the four waves of a workgroup each multiply the WHOLE tile over a quarter of K (wave w
+//     takes the 64-deep units w, w+4, ... of K, so the workgroup as a whole walks 512
+//     contiguous bytes of every row) and every fragment read from LDS feeds MI (or NI) MFMAs;
+//   * each wave has a private ring in LDS, filled by its own direct-to-LDS buffer loads and
+//     drained by its own MFMAs: a wave waits only on its own `vmcnt`, there is no barrier in
+//     the loop;
+//   * a ring stage is one unit: (BM + BN) rows of 128 bytes, XOR-swizzled.  One load
+//     instruction fills 8 rows: lane l lands on 16-byte position l & 7 of row l >> 3 and fetches
+//     chunk (l & 7) ^ ((row >> 1) & 7) of the row, so that the fragment read (lane l: row
+//     l & 15, chunk 4*slice + (l >> 4) -- the operand layout of v_mfma_f32_16x16x32) touches
+//     every bank once.  Whole 128-byte lines per request matter: an L2 delivers whole lines,
+//     and with 64-byte rows (a ring of half units, twice as deep) this kernel ran at half the
+//     rate (1024 x 1024 x 4096 on 64 x 64 tiles: 24.3 us);
+//   * all fragments of a unit are read into registers first, so its stage takes the next
+//     request before the MFMAs start: a ring of NS stages keeps NS units in flight.  (A K loop
+//     software-pipelined by hand -- fragment reads and requests dealt out between the MFMAs --
+//     was 10-35 % slower than this plain order, which the compiler schedules itself);
+//   * every workgroup walks K from its start: the workgroups of an XCD that share rows of A
+//     or B then ask for them at about the same time and all but the first hit in the L2 (a
+//     rotated start per workgroup, as the decode kernels use against HBM channel crowding,
+//     cost 1024 x 1024 x 4096 a third: 14.8 -> 19.8 us);
+//   * the four partial tiles are added in wave order through LDS (a fixed order: results are
+//     reproducible), scaled, rounded once and stored with 8-byte stores.
+// The kernel is bound by what a CU can pull through its L1 ((BM + BN) x 128 bytes per unit of
+// K), which is why the tile is as square as the shape allows.
+// Rows of A past M and rows of B past N are never fetched (the buffer descriptors end at the
+// last valid row of the tile).  Preconditions, checked by the launcher's caller: K % 64 == 0,
+// N % 4 == 0, 16-byte aligned A and B rows, 8-byte aligned C.
+// The reference has no counterpart: its kernels use one tile size (matmul_utils.cuh:362).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "gemm_kernel.hpp"
+#include "gemm_mfma16_kernel.hpp"   // mfma_16x16x32
+#include "splitk_common.hpp"        // DecodeArgs
+
+namespace mi {
+
+template <int BM_, int BN_, int NS_, int DT_>
+struct WaveKConfig {
+    static constexpr int BM = BM_, BN = BN_, NS = NS_, DT = DT_;
+    static constexpr int NT = 256, NW = 4;
+    static constexpr int MI = BM / 16, NI = BN / 16;
+    static constexpr int L = (BM + BN) / 8;                  // load instructions per unit
+    static constexpr int STAGE = (BM + BN) * 128;            // bytes of a ring stage
+    static constexpr int RING = NS * STAGE;
+    static constexpr int PITCH = BN + 4;                     // floats per row of a partial tile (bank spread)
+    static constexpr int PART = BM * PITCH * 4;
+    static constexpr int REGION = RING > PART ? RING : PART; // one wave's share of LDS
+    static constexpr int LDS_BYTES = NW * REGION;
+    static constexpr int QUADS = BM * BN / 4 / NT;           // 4-element groups of C per thread
+    static_assert(BM % 16 == 0 && BN % 16 == 0, "whole 16x16 MFMA tiles");
+    static_assert(NS >= 2 && (NS - 1) * L <= 63, "vmcnt is a 6-bit counter");
+    static_assert(BM * BN / 4 % NT == 0, "the C tile divides over the threads");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
+};
+
+template <class Cfg>
+__global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::NS, DT = Cfg::DT;
+    constexpr int MI = Cfg::MI, NI = Cfg::NI, L = Cfg::L, STAGE = Cfg::STAGE;
+    constexpr int PITCH = Cfg::PITCH, REGION = Cfg::REGION;
+
+    __shared__ __attribute__((aligned(128))) unsigned char lds[Cfg::LDS_BYTES];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int M = p.M, N = p.N, K = p.K;
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    int tm, tn;
+    tile_of_block<4>(blockIdx.x, gridDim.x, tiles_m, tiles_n, tm, tn);
+    const int row0 = tm * BM, col0 = tn * BN;
+    const int KT = K / 64;                                   // units of K
+    const int cnt = (KT - wave + 3) / 4;                     // units of this wave: wave, wave+4, ...
+
+    const int rowsA = (M - row0) < BM ? (M - row0) : BM;
+    const int rowsB = (N - col0) < BN ? (N - col0) : BN;
+    const unsigned char* Ab = (const unsigned char*)p.A + (size_t)row0 * p.lda * 2;
+    const unsigned char* Bb = (const unsigned char*)p.B + (size_t)col0 * p.ldb * 2;
+    const uint32_t bytesA = (uint32_t)((rowsA - 1) * p.lda + K) * 2u;
+    const uint32_t bytesB = (uint32_t)((rowsB - 1) * p.ldb + K) * 2u;
+    const __amdgpu_buffer_rsrc_t rsrcA = __builtin_amdgcn_make_buffer_rsrc((void*)Ab, 0, (int)bytesA, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrcB = __builtin_amdgcn_make_buffer_rsrc((void*)Bb, 0, (int)bytesB, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrcNone = __builtin_amdgcn_make_buffer_rsrc((void*)Ab, 0, 0, 0x00020000);
+
+    const uint32_t ring_base =
+        (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds + (uint32_t)wave * REGION;
+    auto dma = [&](const __amdgpu_buffer_rsrc_t& rsrc, uint32_t voff, uint32_t dst) __attribute__((always_inline)) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                     :: "s"(dst), "v"(voff), "s"(rsrc) : "memory");
+    };
+    auto swz = [](int row) __attribute__((always_inline)) { return (row >> 1) & 7; };
+    // this lane's byte offset inside A and B for load instruction q of a unit (stage rows: A
+    // first, then B; k offset added per request)
+    const int lr = lane >> 3, lc = lane & 7;
+    uint32_t voff[L];
+#pragma unroll
+    for (int q = 0; q < L; ++q) {
+        const int row = q * 8 + lr;
+        const int chunk = lc ^ swz(row);
+        voff[q] = q * 8 < BM ? (uint32_t)(row * p.lda + chunk * 8) * 2u
+                             : (uint32_t)((row - BM) * p.ldb + chunk * 8) * 2u;
+    }
+
+    // unit i of this wave is unit wave + 4*i of the matrix; `rq_gs` follows the unit about to
+    // be requested (requests past the last one fetch nothing), `rq_left` the live units left
+    int rq_gs = wave;
+    int rq_left = cnt;
+    auto request = [&](int stage) __attribute__((always_inline)) {
+        const bool live = rq_left > 0;
+        --rq_left;
+        const uint32_t kb = (uint32_t)rq_gs * 128u;
+        rq_gs += 4;
+        const uint32_t dst = ring_base + (uint32_t)(stage * STAGE);
+#pragma unroll
+        for (int q = 0; q < L; ++q)
+            dma(live ? (q * 8 < BM ? rsrcA : rsrcB) : rsrcNone, voff[q] + kb, dst + (uint32_t)(q * 1024));
+    };
+
+    // fragment read: lane holds row l & 15 of a 16-row block, chunk 4*slice + (l >> 4)
+    const int l16 = lane & 15, q4 = lane >> 4;
+    int rd_off[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) rd_off[ks] = l16 * 128 + ((((ks << 2) | q4) ^ swz(l16)) << 4);
+
+    f32x4_t acc[MI][NI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) acc[i][j] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+#pragma unroll
+    for (int i = 0; i < NS; ++i) request(i);
+
+    const unsigned char* ring = lds + wave * REGION;
+    int s = 0;
+    for (int u = 0; u < cnt; ++u) {
+        // unit u of this wave has landed
+        asm volatile("s_waitcnt vmcnt(%0)" :: "n"((NS - 1) * L) : "memory");
+        const unsigned char* st = ring + s * STAGE;
+        u32x4_t fa[2][MI], fb[2][NI];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+            for (int i = 0; i < MI; ++i) fa[ks][i] = *(const u32x4_t*)(st + i * 2048 + rd_off[ks]);
+#pragma unroll
+            for (int j = 0; j < NI; ++j) fb[ks][j] = *(const u32x4_t*)(st + (BM + j * 16) * 128 + rd_off[ks]);
+        }
+        // its fragments are in registers: the stage takes the request NS units ahead
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        request(s);
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int j = 0; j < NI; ++j) acc[i][j] = mfma_16x16x32<DT>(fb[ks][j], fa[ks][i], acc[i][j]);
+        s = s + 1 == NS ? 0 : s + 1;
+    }
+    // requests past this wave's last unit (empty descriptor: zeros) are still heading for
+    // the ring: drain before the partial tile takes its place
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+
+    // ---- add the four partial tiles in wave order, scale, round, store ----
+    // acc[i][j][e] of lane l is P[m][n], m = i*16 + (l & 15), n = j*16 + 4*(l >> 4) + e
+    float* part = (float*)(lds + wave * REGION);
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+            *(f32x4_t*)(part + (i * 16 + l16) * PITCH + j * 16 + 4 * q4) = acc[i][j];
+    __syncthreads();
+    const bool scaled = p.alpha != 1.0f || p.beta != 0.0f;
+#pragma unroll
+    for (int it = 0; it < Cfg::QUADS; ++it) {
+        const int q = it * 256 + tid;
+        const int m = q / (BN / 4), n = (q % (BN / 4)) * 4;
+        f32x4_t sum = *(const f32x4_t*)((const float*)lds + m * PITCH + n);
+#pragma unroll
+        for (int w = 1; w < 4; ++w) {
+            const f32x4_t v = *(const f32x4_t*)((const float*)(lds + w * REGION) + m * PITCH + n);
+            sum[0] += v[0]; sum[1] += v[1]; sum[2] += v[2]; sum[3] += v[3];
+        }
+        if (scaled) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sum[e] = mul_add_unfused(sum[e], p.alpha, p.beta);
+        }
+        if (row0 + m < M && col0 + n < N) {                  // N % 4 == 0 is a launch precondition
+            u32x2_t w2;
+            w2[0] = cvt_store2<DT>(sum[0], sum[1]);
+            w2[1] = cvt_store2<DT>(sum[2], sum[3]);
+            *(u32x2_t*)((unsigned char*)p.C + ((size_t)(row0 + m) * p.ldc + col0 + n) * 2) = w2;
+        }
+    }
+}
+
+template <class Cfg>
+hipError_t launch_wavek_kernel(const DecodeArgs& a, hipStream_t stream) {
+    const int tiles = ((a.M + Cfg::BM - 1) / Cfg::BM) * ((a.N + Cfg::BN - 1) / Cfg::BN);
+    return launch_kernel(gemm_wavek_kernel<Cfg>, dim3(tiles), dim3(256), stream, a);
+}
+
+}  // namespace mi

@@ -293,6 +293,7 @@ int tuned_config(int M, int N, int K, bool streamable) {
         if (t.M != M || t.N != N || t.K != K) continue;
         const mi::KernelEntry& e = mi::kKernels[t.config];
         if ((is_split_k_decode(e.kind) || e.kind == mi::KIND_STREAM) && (!streamable || M > e.BM)) continue;
+        if (e.kind == mi::KIND_WAVEK && !streamable) continue;
         return t.config;
     }
     return -1;
@@ -345,7 +346,10 @@ int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const vo
     int rc = check_args(config, dtype, M, N, K, A, B, C);
     if (rc != MI_OK) return rc;
     const bool streamable = shape_is_streamable(M, N, K, A, B, C);
-    const Choice choice = choose(config, M, N, K, streamable, shape_is_splittable(N, C, DB),
+    // with a trace buffer the automatic choice stays with the kernels that fill it (the tiled
+    // ones); an explicitly requested decode or small-tile kernel runs and leaves it untouched
+    const Choice choice = choose(config, M, N, K, streamable && !(config == MI_CONFIG_AUTO && DB),
+                                 shape_is_splittable(N, C, DB),
                                  aligned16(A) && aligned16(B) && aligned16(C));
     config = choice.config;
     const mi::KernelEntry& e = mi::kKernels[config];
@@ -375,6 +379,15 @@ int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const vo
             return fail(MI_ERR_UNSUPPORTED,
                         "config %s needs M <= %d, N %% 4 == 0, K %% 64 == 0 and 16-byte aligned operands",
                         e.name, e.BM);
+        hipError_t err = e.launch[dtype][0](args, (hipStream_t)stream);
+        if (err != hipSuccess)
+            return fail(MI_ERR_HIP, "launch of %s failed: %s", e.name, hipGetErrorString(err));
+        return MI_OK;
+    }
+    if (e.kind == mi::KIND_WAVEK) {
+        if (!streamable)
+            return fail(MI_ERR_UNSUPPORTED,
+                        "config %s needs N %% 4 == 0, K %% 64 == 0 and 16-byte aligned operands", e.name);
         hipError_t err = e.launch[dtype][0](args, (hipStream_t)stream);
         if (err != hipSuccess)
             return fail(MI_ERR_HIP, "launch of %s failed: %s", e.name, hipGetErrorString(err));
@@ -466,6 +479,7 @@ int mi_gemm_config_supports(int config, int dtype, int M, int N, int K) {
     const mi::KernelEntry& e = mi::kKernels[config];
     if (is_split_k_decode(e.kind) || e.kind == mi::KIND_STREAM)
         return M <= e.BM && N % 4 == 0 && K % 64 == 0;
+    if (e.kind == mi::KIND_WAVEK) return N % 4 == 0 && K % 64 == 0;
     return e.launch[dtype][1] != nullptr;
 }
 
@@ -479,6 +493,7 @@ int mi_gemm_config_grid(int config, int M, int N, int K) {
         return tiles_n * choose_splits(tiles_n, K, compute_units());
     }
     const int tiles = ((M + e.BM - 1) / e.BM) * ((N + e.BN - 1) / e.BN);
+    if (e.kind == mi::KIND_WAVEK) return K % 64 != 0 ? 0 : tiles;
     if (e.kind == mi::KIND_MFMA16) {   // split-K pieces, assuming an aligned C and no trace buffer
         int kps = K;
         return tiles * choose_tile_splits(e, M, N, K, N % 4 == 0, true, compute_units(), &kps);

@@ -271,7 +271,7 @@ def tune_library_choice(shapes, out_file: Optional[str] = None, margin: float = 
 
     import h100_gemm_amd as mi
     lib = mi._lib.load()
-    cands = [i for i, c in enumerate(kc.CONFIGS) if c.get("EFF") or c["KIND"] in ("stream", "decode")]
+    cands = [i for i, c in enumerate(kc.CONFIGS) if c.get("EFF") or c["KIND"] in ("stream", "decode", "wavek")]
 
     def time_config(config, params, launches):
         for i in range(max(3, launches // 4)):

@@ -15,7 +15,9 @@ template takes (matmul_h100.cu.jinja:9-14) -- re-cast for CDNA4:
              "mfma16" / "ring16" (the same two pipelines on the 16x16x32 MFMA with eight
              or four waves, csrc/gemm_mfma16_kernel.hpp), "decode" (split-K kernel for decode
              shapes, M <= BM, whose LDS ring holds B only, csrc/gemm_decode_kernel.hpp) or
-             "stream" (single-pass decode kernel, csrc/gemm_stream_kernel.hpp)
+             "stream" (single-pass decode kernel, csrc/gemm_stream_kernel.hpp), "wavek" (small
+             tiles with K split over the waves of a workgroup, for outputs of few tiles with a
+             long K, csrc/gemm_wavek_kernel.hpp)
     EPI      1: C tile transposed through LDS and written 16 bytes per lane, 0: 8-byte stores
     DRAIN    (mfma16, optional) d > 0: a second barrier early in each K step (4*d MFMAs after the
              fragment reads) frees the current LDS stage, so the next loads are spread over most
@@ -24,6 +26,9 @@ template takes (matmul_h100.cu.jinja:9-14) -- re-cast for CDNA4:
              register-staged predicated kernel runs best with eight waves)
     EFF      (optional) per-CU throughput relative to the 256x256 tile, measured at 8192^3;
              configs that carry it are the candidates of the automatic shape -> kernel choice
+    WK       (wavek, optional) time model in microseconds: fixed + rounds of workgroups x (per
+             round + K/64 x per unit), least-squares fit on 65 shapes with M, N <= 2048;
+             configs that carry it join the automatic choice
     EFF_E    (optional) throughput of the predicated variant relative to the aligned one, from
              7000^3, 6000^3 and 5000^3 (default 0.85); used for shapes the aligned variant cannot run
 
@@ -48,6 +53,8 @@ def config_name(c: dict) -> str:
         return f"s{c['BM']}x{c['BN']}_n{c['NS']}"
     if c["KIND"] == "decode":
         return f"d{c['BM']}x{c['BN']}_n{c['NS']}"
+    if c["KIND"] == "wavek":
+        return f"k{c['BM']}x{c['BN']}_n{c['NS']}"
     name = (f"t{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_s{c['SWZ']}_g{c['GROUP']}"
             f"_o{c['OCC']}_d{c['DTL']}_e{c['EPI']}")
     if (c.get("EWM", c["WM"]), c.get("EWN", c["WN"])) != (c["WM"], c["WN"]):
@@ -56,7 +63,7 @@ def config_name(c: dict) -> str:
 
 
 def threads(c: dict) -> int:
-    return 256 if c["KIND"] in ("stream", "decode") else c["WM"] * c["WN"] * 64
+    return 256 if c["KIND"] in ("stream", "decode", "wavek") else c["WM"] * c["WN"] * 64
 
 
 def lds_bytes(c: dict) -> int:
@@ -66,6 +73,8 @@ def lds_bytes(c: dict) -> int:
         return 4 * c["NS"] * (c["BM"] + c["BN"]) * 128
     if c["KIND"] == "decode":
         return c["NS"] * c["BN"] * 128
+    if c["KIND"] == "wavek":     # per wave: the ring, or the padded fp32 partial tile if that is larger
+        return 4 * max(c["NS"] * (c["BM"] + c["BN"]) * 128, c["BM"] * (c["BN"] + 4) * 4)
     return 2 * (c["BM"] + c["BN"]) * 128
 
 
@@ -93,6 +102,13 @@ def is_valid_config(c: dict) -> bool:
         return (c["BM"] in (64, 128) and c["BN"] % 32 == 0 and c["NS"] >= 3
                 and (c["NS"] - 1) * (c["BM"] // 32 + c["BN"] // 32) <= 63
                 and lds_bytes(c) <= 160 * 1024)
+    if c["KIND"] == "wavek":
+        # per wave and ring stage (BM + BN) / 8 direct-to-LDS loads, NS stages outstanding
+        return (c["BM"] % 16 == 0 and c["BN"] % 16 == 0 and c["NS"] >= 2
+                and (c["NS"] - 1) * ((c["BM"] + c["BN"]) // 8) <= 63
+                and c["BM"] * c["BN"] // 4 % 256 == 0
+                and (c["BM"] // 16) * (c["BN"] // 16) * 4 <= 256
+                and lds_bytes(c) * c.get("OCC", 1) <= 160 * 1024)
     nt = c["WM"] * c["WN"] * 64
     if nt > 1024 or nt < 64:
         return False
@@ -179,6 +195,13 @@ def _s(BM, NS):
     return dict(KIND="stream", BM=BM, BN=32, NS=NS)
 
 
+def _k(BM, BN, NS, WK=None):
+    c = dict(KIND="wavek", BM=BM, BN=BN, NS=NS)
+    if WK is not None:
+        c["WK"] = WK
+    return c
+
+
 def _d(BM, NS, BN=128):
     return dict(KIND="decode", BM=BM, BN=BN, NS=NS)
 
@@ -217,6 +240,10 @@ CONFIGS = [
     _m(192, 128, 2, 2, DRAIN=1, EFF=0.74, EFF_E=0.85),
     _d(128, NS=3),
     _d(64, NS=4),
+    _k(32, 32, NS=4, WK=(0.82, 1.70, 0.0827)),
+    _k(64, 32, NS=3, WK=(0.80, 2.09, 0.1203)),
+    _k(64, 64, NS=2, WK=(0.46, 3.09, 0.1655)),
+    _k(96, 64, NS=2, WK=(1.04, 4.38, 0.2317)),
 ]
 
 assert all(is_valid_config(c) for c in CONFIGS), [config_name(c) for c in CONFIGS if not is_valid_config(c)]

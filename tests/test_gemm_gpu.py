@@ -180,6 +180,45 @@ def test_decode_kernels(mi, orc, config):
         Dev(mi, A, B, 8, 256).run(100, config=config)
 
 
+# ------------------------- small tiles, K split over the waves of a workgroup (few tiles, long K) ----
+
+@pytest.mark.parametrize("config", all_configs(("wavek",)))
+def test_wave_split_k_kernels(mi, orc, config):
+    from h100_gemm_amd import kernel_configs as kc
+    bm, bn = kc.CONFIGS[config]["BM"], kc.CONFIGS[config]["BN"]
+    # whole tiles, ragged M and N (rows past M / N are never fetched nor stored), one tile, a
+    # single K unit (three of the four waves have nothing to add), K units that do not divide
+    # over the waves, several rounds of workgroups
+    for M, N, K in [(512, 512, 4096), (bm, bn, 64), (bm + 1, bn + 4, 128), (1, 4, 64), (100, 36, 192),
+                    (777, 1000, 320), (1536, 1536, 1536), (33, 8, 448), (2 * bm - 1, 5 * bn - 4, 2112)]:
+        check(mi, orc, M, N, K, "int", config=config, exact=True)     # sums of exact ints: any order gives the oracle's bits
+    check(mi, orc, 1024, 1024, 4096, "uniform", config=config)
+    check(mi, orc, 512, 768, 2048, "normal", config=config, dtype=orc.FP16)
+    check_epilogue(mi, orc, 300, 260, 1024, "int", -0.5, 2.75, config=config, exact=True)
+    check_epilogue(mi, orc, 512, 512, 4096, "uniform", 0.37, 1.25, config=config)
+    check_epilogue(mi, orc, 200, 132, 1024, "int", 2.0, -1.0, config=config, c_layout=mi.MI_C_COL_MAJOR, exact=True)
+    # shapes the kernel cannot run are refused, not mis-computed
+    for M, N, K in [(256, 256, 100), (256, 254, 128)]:
+        A, B = make_inputs(orc, M, N, K, "int")
+        with pytest.raises(mi.MiGemmError) as ei:
+            Dev(mi, A, B, M, N).run(K, config=config)
+        assert ei.value.code == mi._lib.MI_ERR_UNSUPPORTED
+
+
+def test_wave_split_k_dispatch_and_determinism(mi, orc):
+    from h100_gemm_amd import kernel_configs as kc
+    # the automatic choice for few-tile shapes; the same answers as the tiled kernels where
+    # its preconditions fail (K % 64, N % 4)
+    for M, N, K in [(512, 512, 4096), (1024, 1024, 4096), (512, 512, 4100), (512, 510, 4096), (640, 384, 3328)]:
+        check(mi, orc, M, N, K, "int", exact=True)
+    assert kc.CONFIGS[mi.select_config(512, 512, 4096)]["KIND"] == "wavek"
+    A, B = make_inputs(orc, 1024, 1024, 4096, "uniform")
+    d = Dev(mi, A, B, 1024, 1024)
+    C0 = d.run(4096)
+    for _ in range(3):
+        assert (d.run(4096) == C0).all()          # fixed summation order: bit-reproducible
+
+
 def test_decode_dispatch_and_determinism(mi, orc):
     # automatic choice: decode kernel when its preconditions hold, the predicated tile kernel
     # otherwise -- same answers either way
@@ -620,24 +659,38 @@ def test_reference_gpu_gemm_is_bit_identical_to_the_oracle(mi, orc):
 # ------------------------------------------------------------------ trace buffer ------
 
 def test_db_trace_records(mi, orc):
+    from h100_gemm_amd import kernel_configs as kc
     M = N = K = 1024
     A, B = make_inputs(orc, M, N, K, "int")
     d = Dev(mi, A, B, M, N)
     words = mi._lib.load().mi_gemm_trace_words(M, N, K)
     dDB = mi.DeviceBuffer(words * 4)
-    dDB.fill_bytes(0xFF)
-    cfg = mi.select_config(M, N, K)
-    C = d.run(K, DB=dDB)
-    assert (C == orc.reference_cpu_gemm(A, B)).all()        # tracing must not change results
-    db = dDB.to_numpy((words,), np.int32)
-    n = 0
-    while n + 5 < words and db[n] != -1:
-        n += 6
-    rec = db[:n].reshape(-1, 6)
-    assert len(rec) == mi.config_grid(cfg, M, N, K)
+
+    def records(config):
+        dDB.fill_bytes(0xFF)
+        C = d.run(K, config, DB=dDB)
+        assert (C == orc.reference_cpu_gemm(A, B)).all()        # tracing must not change results
+        db = dDB.to_numpy((words,), np.int32)
+        n = 0
+        while n + 5 < words and db[n] != -1:
+            n += 6
+        assert db[n] == -1
+        return db[:n].reshape(-1, 6)
+
+    cfg = mi.find_config("m128x128_w2x2_g4_b1_o2")
+    rec = records(cfg)
+    assert len(rec) == mi.config_grid(cfg, M, N, K) == 64
     assert (rec[:, 3] == K // 64).all() and (rec[:, 5] == 1).all()
     assert (rec[:, 2] > 0).all() and (rec[:, 0] >= 0).all() and (rec[:, 0] < rec[:, 2]).all()
-    assert db[n] == -1
+    # the automatic choice for this shape is a small-tile kernel, which keeps no records: with
+    # a trace buffer it stays with the tiled kernels
+    assert kc.CONFIGS[mi.select_config(M, N, K)]["KIND"] == "wavek"
+    rec = records(mi.MI_CONFIG_AUTO)
+    tiled = [i for i, c in enumerate(kc.CONFIGS) if c["KIND"] == "mfma16" and c.get("EFF")]
+    assert len(rec) in {-(-M // kc.CONFIGS[i]["BM"]) * -(-N // kc.CONFIGS[i]["BN"]) for i in tiled}
+    assert (rec[:, 3] == K // 64).all()
+    # asked for by name, the small-tile kernel runs and leaves the buffer untouched
+    assert len(records(mi.select_config(M, N, K))) == 0
 
 
 # --------------------------------------------------------------- C++ harness ----------

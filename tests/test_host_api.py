@@ -137,6 +137,13 @@ def test_config_table(mi):
             assert L.mi_gemm_config_supports(i, 0, 16, 8190, 8192) == 0
             assert mi.config_grid(i, 16, 8192, 8192) >= 64
             assert mi.config_grid(i, c["BM"] + 1, 8192, 8192) == 0
+        elif c["KIND"] == "wavek":
+            # any M; whole 64-deep K units, N a multiple of 4; no ragged twin
+            assert mi.config_grid(i, 1000, 780, 64) == -(-1000 // c["BM"]) * -(-780 // c["BN"])
+            assert L.mi_gemm_config_supports(i, 0, 1000, 780, 4096) == 1
+            assert L.mi_gemm_config_supports(i, 0, 1000, 780, 4100) == 0
+            assert L.mi_gemm_config_supports(i, 0, 1000, 778, 4096) == 0
+            assert mi.config_grid(i, 1000, 780, 4100) == 0
         else:
             tiles = -(-1000 // c["BM"]) * -(-777 // c["BN"])
             assert mi.config_grid(i, 1000, 777, 64) == tiles
@@ -156,26 +163,35 @@ def test_config_table(mi):
         assert mi.config_name(mi.select_config(M, N, K)) == name
     assert kc.CONFIGS[mi.select_config(8192, 8192, 8192)]["KIND"] == "mfma16"
     assert kc.CONFIGS[mi.select_config(4096, 4096, 4096)]["KIND"] == "mfma16"
+    # few tiles and a long K: small tiles with K split over the waves, when the kernel can run the shape
+    assert kc.CONFIGS[mi.select_config(512, 512, 4096)]["KIND"] == "wavek"
+    assert kc.CONFIGS[mi.select_config(1024, 1024, 4096)]["KIND"] == "wavek"
+    assert kc.CONFIGS[mi.select_config(512, 512, 4100)]["KIND"] == "mfma16"
+    assert kc.CONFIGS[mi.select_config(512, 510, 4096)]["KIND"] == "mfma16"
     # wave quantisation: 256 CUs; 8192^2 fills four rounds of 256x256 tiles, 4095x6143 fills
     # two rounds of 256x192 tiles exactly (256x256 would leave half of the second round
-    # idle), and 512^2 is a single partial round whatever the tile, so the smallest wins
+    # idle), and 512^2 is a single partial round whatever the tiled kernel: the small-tile
+    # kernel gives every CU a 32x32 tile (one with a ragged K cannot run it: 128x128 tiles)
     def picked(M, N, K):
         c = kc.CONFIGS[mi.select_config(M, N, K)]
         return c["BM"], c["BN"]
     assert picked(8192, 8192, 8192) == (256, 256)
     assert picked(8192, 28672, 8192) == (256, 256)
     assert picked(4095, 6143, 3073) == (256, 192)
-    assert picked(512, 512, 512) == (128, 128)
-    assert kc.CONFIGS[mi.select_config(512, 512, 512)]['KIND'] == 'mfma16'
-    assert all("EFF" in kc.CONFIGS[mi.select_config(M, N, 4096)] for M in (257, 1000, 5000) for N in (100, 3000))
+    assert picked(512, 512, 512) == (32, 32)
+    assert kc.CONFIGS[mi.select_config(512, 512, 512)]['KIND'] == 'wavek'
+    assert picked(512, 512, 520) == (128, 128)
+    assert kc.CONFIGS[mi.select_config(512, 512, 520)]['KIND'] == 'mfma16'
+    assert all("EFF" in kc.CONFIGS[mi.select_config(M, N, 4100)] for M in (257, 1000, 5000) for N in (100, 3000))
     # few tiles and a long K: split-K pieces of a tiled kernel fill the CUs
     c = mi.select_config(256, 8192, 8192)
     assert kc.CONFIGS[c]["KIND"] == "mfma16" and (kc.CONFIGS[c]["BM"], kc.CONFIGS[c]["BN"]) == (256, 128)
     assert 128 < mi.config_grid(c, 256, 8192, 8192) <= 256          # 64 tiles x 3 or 4 pieces
-    c = mi.select_config(512, 512, 4096)
+    c = mi.find_config("m128x128_w2x2_g4_b1_o2")                    # (the automatic choice is the small-tile kernel)
     assert mi.config_grid(c, 512, 512, 4096) == 16 * 8              # 128x128 tiles x 8 pieces of 512
     assert mi.config_grid(mi.select_config(8192, 8192, 8192), 8192, 8192, 8192) == 1024   # no split-K when the tiles fill the chip
-    assert mi.config_grid(mi.select_config(512, 512, 512), 512, 512, 512) == 16           # nor for a short K
+    assert mi.config_grid(mi.select_config(512, 512, 520), 512, 512, 520) == 16           # nor for a short K
+    assert mi.config_grid(mi.select_config(512, 512, 512), 512, 512, 512) == 256          # 32x32 tiles, one per CU
     c = mi.select_config(512, 510, 4096)
     assert mi.config_grid(c, 512, 510, 4096) == -(-512 // kc.CONFIGS[c]["BM"]) * -(-510 // kc.CONFIGS[c]["BN"])   # N % 4 != 0: no split-K
     assert "EFF" in kc.CONFIGS[mi.select_config(200, 8190, 8192)]        # N % 4 != 0: tiled
@@ -299,7 +315,7 @@ def test_tuned_shapes_file_overrides_the_model(mi, tmp_path):
     assert out.returncode == 0, out.stderr
     lines = out.stdout.split()
     assert lines[0] == "4"                                   # four lines name a compiled configuration
-    assert lines[1:] == ["m256x256_w2x2_g8_b1", "m256x192_w2x2_g4_b3", "m128x128_w2x2_g4_b1_o2",
+    assert lines[1:] == ["m256x256_w2x2_g8_b1", "m256x192_w2x2_g4_b3", "k32x32_n4",
                          "m256x256_w2x2_g4_b3", "s64x32_n3", "m256x256_w2x2_g4_b3"], lines
     assert mi._lib.load().mi_gemm_tuned_entries() == 0       # this process has no such file
 

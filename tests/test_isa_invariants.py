@@ -25,8 +25,8 @@ def test_m0_is_only_written_by_the_kernels_own_asm():
     """Consecutive direct-to-LDS loads share one M0 value across asm statements, so nothing
     the compiler emits in between may write M0; and every load that follows a write of M0
     directly is preceded by the wait state the hardware needs."""
-    units = built_units(("mfma16", "decode", "stream"))
-    assert len(units) >= 12
+    units = built_units(("mfma16", "decode", "stream", "wavek"))
+    assert len(units) >= 16
     for name, c, text in units:
         n = isa_check.check_m0(name, text, need_kernels=8 if c["KIND"] == "mfma16" else 1)
         assert n >= (8 if c["KIND"] == "mfma16" else 2), (name, n)
