@@ -37,12 +37,14 @@ WORKLOADS = {
     "square512": (512, 512, 512, "uniform"),
     "square8192": (8192, 8192, 8192, "uniform"),
     "mlp_up": (8192, 28672, 8192, "normal"),
-    "mlp_up": ("m256x256_w2x2_g4_b3", (2753408 * 2.0 + 458779) * 1024),         # 6.1 GB against 1.34 GB algorithmic
     "mlp_down": (8192, 8192, 28672, "normal"),
     "skinny16": (16, 8192, 8192, "normal"),
     "skinny64": (64, 8192, 8192, "normal"),
     "skinny128": (128, 8192, 8192, "normal"),
     "unaligned": (4095, 6143, 3073, "uniform"),
+    # outputs of few tiles (not BASELINE configurations; for the profiles of the small-tile kernel)
+    "fewtile512": (512, 512, 4096, "uniform"),
+    "fewtile1024": (1024, 1024, 4096, "uniform"),
 }
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (the summaries under
 # profiles/ give the commands), scaled by the same counters on a copy kernel of known size:

@@ -319,3 +319,22 @@ def test_tuned_shapes_file_overrides_the_model(mi, tmp_path):
                          "m256x256_w2x2_g4_b3", "s64x32_n3", "m256x256_w2x2_g4_b3"], lines
     assert mi._lib.load().mi_gemm_tuned_entries() == 0       # this process has no such file
 
+
+
+def test_bench_tables_are_well_formed(mi):
+    """bench.py's workload table names shapes and fills; its profile constants name a compiled
+    configuration each and only workloads that exist; more than one GPU is refused."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("bench_module", ROOT / "bench.py")
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    for name, w in bench.WORKLOADS.items():
+        M, N, K, fill = w
+        assert all(isinstance(v, int) and v > 0 for v in (M, N, K)) and fill in ("uniform", "normal", "int"), name
+        assert 0 <= mi.select_config(M, N, K) < mi.num_configs()
+    for name in ("square512", "square8192", "mlp_up", "mlp_down", "skinny16", "skinny64", "skinny128", "unaligned"):
+        assert name in bench.WORKLOADS                   # the BASELINE configurations
+    for name, (config, nbytes) in bench.MEASURED_TRAFFIC_BYTES.items():
+        assert name in bench.WORKLOADS and mi.find_config(config) >= 0 and nbytes > 0, name
+    out = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"], capture_output=True, text=True, cwd=ROOT)
+    assert out.returncode == 2 and "ONE GPU" in out.stderr
