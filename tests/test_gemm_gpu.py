@@ -194,6 +194,10 @@ def test_wave_split_k_kernels(mi, orc, config):
         check(mi, orc, M, N, K, "int", config=config, exact=True)     # sums of exact ints: any order gives the oracle's bits
     check(mi, orc, 1024, 1024, 4096, "uniform", config=config)
     check(mi, orc, 512, 768, 2048, "normal", config=config, dtype=orc.FP16)
+    # hundreds of thousands of tile rows / columns (64-bit row offsets), the longest K the library takes
+    check(mi, orc, 600000, 8, 128, "int", config=config, exact=True)
+    check(mi, orc, 8, 600000, 128, "int", config=config, exact=True)
+    check(mi, orc, 40, 36, 4194240, "uniform", config=config)
     check_epilogue(mi, orc, 300, 260, 1024, "int", -0.5, 2.75, config=config, exact=True)
     check_epilogue(mi, orc, 512, 512, 4096, "uniform", 0.37, 1.25, config=config)
     check_epilogue(mi, orc, 200, 132, 1024, "int", 2.0, -1.0, config=config, c_layout=mi.MI_C_COL_MAJOR, exact=True)
