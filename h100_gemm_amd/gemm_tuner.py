@@ -294,7 +294,7 @@ def tune_library_choice(shapes, out_file: Optional[str] = None, margin: float = 
         A, B = np.resize(block, (M, K)), np.resize(block[::-1], (N, K))
         # decode shapes stream their weights from HBM in real use: enough copies of B to exceed
         # the 256 MB memory-side cache, visited in turn
-        copies = min(8, -(-(600 << 20) // B.nbytes)) if M <= 128 else 1
+        copies = min(8, -(-(600 << 20) // B.nbytes)) if M <= int(os.environ.get('MI_TUNER_ROTATE_B_UP_TO_M', '128')) else 1
         dA, dC = mi.DeviceBuffer.from_numpy(A), mi.DeviceBuffer(M * N * 2)
         dBs = [mi.DeviceBuffer.from_numpy(B) for _ in range(copies)]
         params = [mi.GemmParams(M, N, K, dA, dB, dC) for dB in dBs]

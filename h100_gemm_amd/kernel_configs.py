@@ -224,7 +224,7 @@ CONFIGS = [
     _m(256, 256, 2, 2),
     _m(256, 256, 2, 2, DRAIN=3, EFF=1.0, EFF_E=0.82),
     _m(256, 192, 2, 2, DRAIN=3, EFF=0.89, EFF_E=0.90),
-    _m(128, 256, 2, 2, DRAIN=1, EFF=0.875, EFF_E=0.80),
+    _m(128, 256, 2, 2, DRAIN=1, EFF=0.84, EFF_E=0.80),
     _m(256, 128, 2, 2, DRAIN=1, EFF=0.845, EFF_E=0.80),
     _m(128, 128, 2, 2, DRAIN=1, OCC=2, EFF=0.78, EFF_E=0.74),
     _m(256, 256, 4, 2),
