@@ -58,8 +58,8 @@ MEASURED_TRAFFIC_BYTES = {
     "unaligned": ("m256x192_w2x2_g4_b3", (130105 * 2.0 + 49737) * 1024),       # 0.317 GB against 0.113 GB algorithmic
     "mlp_up": ("m256x256_w2x2_g4_b3", (2753408 * 2.0 + 458779) * 1024),         # 6.1 GB against 1.34 GB algorithmic
     "mlp_down": ("m256x256_w2x2_g8_b1", (2.7535e6 * 2.0 + 131072) * 1024),      # 5.8 GB against 1.07 GB algorithmic
-    "square512": ("k32x32_n4", (1569.0 * 2.0 + 512) * 1024),           # 3.6 MB against 1.5 MB algorithmic: a copy of the rows per L2
-    "fewtile512": ("k32x32_n4", (12321.0 * 2.0 + 512) * 1024),         # 25.8 MB against 8.9 MB algorithmic
+    "square512": ("k32x32_n2", (1569.0 * 2.0 + 512) * 1024),           # 3.6 MB against 1.5 MB algorithmic: a copy of the rows per L2
+    "fewtile512": ("k32x32_n2", (12321.0 * 2.0 + 512) * 1024),         # 25.8 MB against 8.9 MB algorithmic
     "fewtile1024": ("k64x64_n2", (24626.5 * 2.0 + 2048) * 1024),       # 52.5 MB against 18.9 MB algorithmic
     "skinny64": ("d64x128_n4", ((69689 + 4114) * 2.0 + 8192 + 1024) * 1024),     # main + reduce kernels
     "skinny128": ("d128x128_n3", ((73797 + 8210) * 2.0 + 16384 + 2048) * 1024),   # main + reduce kernels

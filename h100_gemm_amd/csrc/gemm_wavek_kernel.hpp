@@ -66,7 +66,7 @@ struct WaveKConfig {
     static constexpr int LDS_BYTES = NW * REGION;
     static constexpr int QUADS = BM * BN / 4 / NT;           // 4-element groups of C per thread
     static_assert(BM % 16 == 0 && BN % 16 == 0, "whole 16x16 MFMA tiles");
-    static_assert(NS >= 2 && (NS - 1) * L <= 63, "vmcnt is a 6-bit counter");
+    static_assert(NS >= 1 && (NS - 1) * L <= 63, "vmcnt is a 6-bit counter");
     static_assert(BM * BN / 4 % NT == 0, "the C tile divides over the threads");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
 };

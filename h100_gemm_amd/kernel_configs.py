@@ -26,9 +26,11 @@ template takes (matmul_h100.cu.jinja:9-14) -- re-cast for CDNA4:
              register-staged predicated kernel runs best with eight waves)
     EFF      (optional) per-CU throughput relative to the 256x256 tile, measured at 8192^3;
              configs that carry it are the candidates of the automatic shape -> kernel choice
-    WK       (wavek, optional) time model in microseconds: fixed + rounds of workgroups x (per
-             round + K/64 x per unit), least-squares fit on 65 shapes with M, N <= 2048;
-             configs that carry it join the automatic choice
+    WK       (wavek, optional) time model in microseconds, (fixed, per round, per unit, per
+             tile): fixed + rounds of co-resident workgroups (tiles / (CUs x OCC), rounded up)
+             x per round + tiles per CU (rounded up) x (per tile + K/64 x per unit);
+             non-negative least squares on 89 shapes; configs that carry it join the
+             automatic choice
     EFF_E    (optional) throughput of the predicated variant relative to the aligned one, from
              7000^3, 6000^3 and 5000^3 (default 0.85); used for shapes the aligned variant cannot run
 
@@ -104,7 +106,7 @@ def is_valid_config(c: dict) -> bool:
                 and lds_bytes(c) <= 160 * 1024)
     if c["KIND"] == "wavek":
         # per wave and ring stage (BM + BN) / 8 direct-to-LDS loads, NS stages outstanding
-        return (c["BM"] % 16 == 0 and c["BN"] % 16 == 0 and c["NS"] >= 2
+        return (c["BM"] % 16 == 0 and c["BN"] % 16 == 0 and c["NS"] >= 1
                 and (c["NS"] - 1) * ((c["BM"] + c["BN"]) // 8) <= 63
                 and c["BM"] * c["BN"] // 4 % 256 == 0
                 and (c["BM"] // 16) * (c["BN"] // 16) * 4 <= 256
@@ -195,8 +197,10 @@ def _s(BM, NS):
     return dict(KIND="stream", BM=BM, BN=32, NS=NS)
 
 
-def _k(BM, BN, NS, WK=None):
+def _k(BM, BN, NS, WK=None, OCC=1):
     c = dict(KIND="wavek", BM=BM, BN=BN, NS=NS)
+    if OCC != 1:
+        c["OCC"] = OCC          # workgroups that fit a CU together (LDS): rounds of the time model
     if WK is not None:
         c["WK"] = WK
     return c
@@ -240,10 +244,12 @@ CONFIGS = [
     _m(192, 128, 2, 2, DRAIN=1, EFF=0.74, EFF_E=0.85),
     _d(128, NS=3),
     _d(64, NS=4),
-    _k(32, 32, NS=4, WK=(0.82, 1.70, 0.0827)),
-    _k(64, 32, NS=3, WK=(0.80, 2.09, 0.1203)),
-    _k(64, 64, NS=2, WK=(0.46, 3.09, 0.1655)),
-    _k(96, 64, NS=2, WK=(1.04, 4.38, 0.2317)),
+    _k(32, 32, NS=1, OCC=5, WK=(2.18, 0.0, 0.0775, 0.314)),
+    _k(32, 32, NS=2, OCC=2, WK=(1.71, 0.153, 0.0753, 0.580)),
+    _k(64, 32, NS=3, WK=(0.87, 2.10, 0.1188, 0.0)),
+    _k(64, 64, NS=1, OCC=2, WK=(1.93, 2.19, 0.1792, 0.0)),
+    _k(64, 64, NS=2, WK=(0.88, 2.81, 0.1648, 0.0)),
+    _k(96, 64, NS=2, WK=(1.35, 4.06, 0.2306, 0.0)),
 ]
 
 assert all(is_valid_config(c) for c in CONFIGS), [config_name(c) for c in CONFIGS if not is_valid_config(c)]
