@@ -67,7 +67,10 @@ def render_sources(configs=None) -> list[Path]:
     for old in GEN.glob("unit_*.hip"):
         if old.name not in keep:
             old.unlink()
-            old.with_suffix(".o").unlink(missing_ok=True)
+            for left in GEN.glob(old.stem + ".*"):          # object, stamp
+                left.unlink()
+            for left in GEN.glob(old.stem + "-hip-*"):      # kept assembly text
+                left.unlink()
     return units
 
 
