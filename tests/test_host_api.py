@@ -339,3 +339,35 @@ def test_bench_tables_are_well_formed(mi):
         assert name in bench.WORKLOADS and mi.find_config(config) >= 0 and nbytes > 0, name
     out = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"], capture_output=True, text=True, cwd=ROOT)
     assert out.returncode == 2 and "ONE GPU" in out.stderr
+
+
+def test_automatic_choice_always_names_a_kernel_that_can_run_the_shape(mi):
+    """For any shape the automatic choice is a configuration that supports it (the decode and
+    small-tile kernels have preconditions on M, N % 4 and K % 64; everything else has a
+    predicated variant) with a non-empty grid -- seeded random shapes over every regime of the
+    choice, and the same answer when asked twice."""
+    import numpy as np
+    from h100_gemm_amd import kernel_configs as kc
+    L = mi._lib.load()
+    rng = np.random.default_rng(20)
+    picks = set()
+    for it in range(4000):
+        kind = it % 5
+        if kind == 0:       # decode
+            M, N, K = rng.integers(1, 129), 4 * rng.integers(1, 8000), 64 * rng.integers(1, 400)
+        elif kind == 1:     # few tiles
+            M, N, K = rng.integers(1, 2049), 4 * rng.integers(1, 513), 64 * rng.integers(1, 257)
+        elif kind == 2:     # arbitrary
+            M, N, K = rng.integers(1, 9000), rng.integers(1, 9000), rng.integers(1, 9000)
+        elif kind == 3:     # large, aligned
+            M, N, K = 256 * rng.integers(1, 40), 256 * rng.integers(1, 120), 128 * rng.integers(1, 230)
+        else:               # extreme aspect ratios
+            M, N, K = rng.choice([1, 3, 100000]), rng.choice([1, 4, 8, 200000]), rng.choice([1, 64, 4096, 100000])
+        M, N, K = int(M), int(N), int(K)
+        c = mi.select_config(M, N, K)
+        assert 0 <= c < mi.num_configs(), (M, N, K, c)
+        assert L.mi_gemm_config_supports(c, 0, M, N, K) == 1, (M, N, K, mi.config_name(c))
+        assert mi.config_grid(c, M, N, K) > 0, (M, N, K, mi.config_name(c))
+        assert mi.select_config(M, N, K) == c
+        picks.add(kc.CONFIGS[c]["KIND"])
+    assert picks >= {"mfma16", "stream", "decode", "wavek"}
