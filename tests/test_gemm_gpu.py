@@ -329,6 +329,30 @@ def test_random_shapes_and_alignments_every_tiled_kind(mi, orc):
         assert (guard == 0xEEEE).all(), "bytes outside C were written"
 
 
+def test_random_shapes_small_tile_and_decode_kinds(mi, orc):
+    # seeded sweep for the kernels that need whole 64-deep K units, N % 4 == 0 and 16-byte aligned
+    # operands: ragged M and N, one to many K units, base pointers at multiples of 16 (A, B) and
+    # 8 (C) bytes, through the automatic choice and through every such configuration that can
+    # run the shape; an odd operand offset must send the automatic choice to a predicated kernel
+    from h100_gemm_amd import kernel_configs as kc
+    rng = np.random.default_rng(20241125)
+    special = [i for i, c in enumerate(kc.CONFIGS) if c["KIND"] in ("wavek", "stream", "decode")]
+    # MI_GEMM_RANDOM_CASES=<n> turns this into a longer sweep (36 cases by default)
+    for it in range(int(os.environ.get("MI_GEMM_RANDOM_CASES", "36"))):
+        M = int(rng.choice([rng.integers(1, 130), rng.integers(1, 700)]))
+        N = 4 * int(rng.integers(1, 180))
+        K = 64 * int(rng.choice([1, 2, 3, rng.integers(4, 40)]))
+        offA, offB, offC = 16 * int(rng.integers(0, 4)), 16 * int(rng.integers(0, 4)), 8 * int(rng.integers(0, 8))
+        able = [i for i in special if mi._lib.load().mi_gemm_config_supports(i, 0, M, N, K)]
+        config = -1 if it % 3 == 0 or not able else able[int(rng.integers(0, len(able)))]
+        if it % 7 == 3:
+            config, offA = -1, offA + 2          # not 16-byte aligned: none of these kernels may be chosen
+        print(f"case {it}: M={M} N={N} K={K} offsets {offA},{offB},{offC} config={config}", flush=True)
+        C, ref, guard = _run_offset(mi, orc, config, M, N, K, offA, offB, offC)
+        assert (C == ref).all(), f"{int((C != ref).sum())} elements differ"
+        assert (guard == 0xEEEE).all(), "bytes outside C were written"
+
+
 def test_non_default_streams_and_host_threads(mi, orc):
     """The ABI's stream argument: two host threads, each launching on a stream of its own
     (created with default priority) and waiting with mi_stream_sync.  The shapes include
