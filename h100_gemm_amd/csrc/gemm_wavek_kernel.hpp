@@ -33,10 +33,14 @@
 //     reproducible), scaled, rounded once and stored with 8-byte stores.
 // The kernel is bound by what a CU can pull through its L1 ((BM + BN) x 128 bytes per unit of
 // K, measured 80-100 GB/s per CU), which is why the tile is as square as the shape allows.
+// Rings of one or two stages leave room for two to five workgroups on a CU (32 x 32 with one
+// stage: 32 KB of LDS); alone on its CU such a workgroup is level with the deep rings, with
+// company it is 5-18 % ahead once the tiles run to more than one round, because co-resident
+// workgroups hide each other's first loads and epilogue (1344^3 on 64 x 64: 13.2 -> 11.3 us).
 // Eight waves (two per SIMD, K split eight ways, rings half as deep) ran level with or up to
-// 8 % behind four on every shape tried: hiding more latency does not help.  Tiles of 128 x 128
-// and 128 x 64 with a single stage per wave (all that fits) were far behind the tiled kernels
-// (2048^3: 26.5 us against 19.6): with one stage, loading and multiplying take turns.
+// 8 % behind four on every shape tried.  Tiles of 128 x 128 and 128 x 64, which fit with a
+// single stage and one workgroup per CU only, were far behind the tiled kernels (2048^3:
+// 26.5 us against 19.6): alone and with one stage, loading and multiplying take turns.
 // Rows of A past M and rows of B past N are never fetched (the buffer descriptors end at the
 // last valid row of the tile).  Preconditions, checked by the launcher's caller: K % 64 == 0,
 // N % 4 == 0, 16-byte aligned A and B rows, 8-byte aligned C.
