@@ -38,20 +38,29 @@ namespace mi {
 
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
-template <int BM_, int BN_, int WM_, int WN_, int GROUP_, int DT_, int DRAIN_ = 0, bool EDGE_ = false, int OCC_ = 1>
+// KG = 2: eight waves as two groups of WM x WN, each multiplying one half of K of the same tile
+// in LDS stages of its own; the groups share the barriers (same trip count: K % 256 == 0) and
+// the second hands its accumulators to the first through LDS at the end.  For tiles that are
+// alone on their CU (a lone 128x128 workgroup of the two-per-CU kernel runs at ~62 % of its
+// paired rate: two waves per SIMD hide each other's LDS and load latency).
+template <int BM_, int BN_, int WM_, int WN_, int GROUP_, int DT_, int DRAIN_ = 0, bool EDGE_ = false, int OCC_ = 1,
+          int KG_ = 1>
 struct Mfma16Config {
     static constexpr int BM = BM_, BN = BN_, BK = 64;
     static constexpr int WM = WM_, WN = WN_, GROUP = GROUP_, DT = DT_;
     static constexpr bool DRAIN = DRAIN_ != 0;
     static constexpr bool EDGE = EDGE_;                  // predicated variant: any M, N, K, any alignment
-    static constexpr int NT = WM * WN * 64, NW = WM * WN;
+    static constexpr int KG = KG_;                       // groups of waves that split K
+    static constexpr int NW = WM * WN, NT = NW * KG * 64;
     static constexpr int TM = BM / WM, TN = BN / WN;
     static constexpr int MI = TM / 16, NI = TN / 16;
-    static constexpr int RPP = NT / 8;                   // tile rows one pass of all threads loads
+    static constexpr int RPP = NW * 8;                   // tile rows one pass of a group's threads loads
     static constexpr int LA = BM / RPP, LB = BN / RPP;   // load instructions per wave per slab
     static constexpr int A_STAGE = BM * 128, B_STAGE = BN * 128;
-    static constexpr int LDS_BYTES = 2 * (A_STAGE + B_STAGE);
+    static constexpr int LDS_GROUP = 2 * (A_STAGE + B_STAGE);
+    static constexpr int LDS_BYTES = KG * LDS_GROUP;
     static constexpr int OCC = OCC_;                     // workgroups per CU the register / LDS budget is sized for
+    static_assert(KG == 1 || (KG == 2 && BM * BN * 4 <= LDS_GROUP), "the second group's accumulators pass through its stages");
     static constexpr int WAVES_PER_EU = NT / 256 * OCC;
     static constexpr int NMMA = MI * NI, NFR = MI + NI;
     static_assert(NT == 256 || NT == 512, "one or two waves per SIMD");
@@ -69,7 +78,7 @@ struct Mfma16Config {
     static constexpr int D0 = DSPD > 0 ? (NMMA - SA - 1 + DSPD - 1) / DSPD : 0;
     static_assert(!DRAIN || (DSPD >= 1 && SA + 1 < NMMA && D0 <= LA + LB), "drain schedule");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
-    static_assert(BM * BN * 2 <= LDS_BYTES, "the epilogue stages the C tile in the stage buffers");
+    static_assert(BM * BN * 2 <= LDS_GROUP, "the epilogue stages the C tile in the stage buffers");
 };
 
 template <int DT>
@@ -102,8 +111,9 @@ gemm_mfma16_kernel(const GemmArgs p) {
     constexpr int NMMA = Cfg::NMMA, NFR = Cfg::NFR, DT = Cfg::DT;
     constexpr int TM = Cfg::TM, TN = Cfg::TN;
 
-    // [A stage 0][A stage 1][B stage 0][B stage 1]
-    __shared__ __attribute__((aligned(128))) unsigned char lds[Cfg::LDS_BYTES];
+    // [A stage 0][A stage 1][B stage 0][B stage 1], once per K group
+    __shared__ __attribute__((aligned(128))) unsigned char lds_all[Cfg::LDS_BYTES];
+    static_assert(!(SPLITK && Cfg::KG > 1), "K is split either over workgroups or over the groups of one");
 
     long long tr_wait = 0, tr_t0 = 0, tr_loop = 0;
     int tr_cnt = 0;
@@ -112,8 +122,16 @@ gemm_mfma16_kernel(const GemmArgs p) {
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_all = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int kg = Cfg::KG > 1 ? wave_all / Cfg::NW : 0;        // K group of this wave
+    const int wave = Cfg::KG > 1 ? wave_all % Cfg::NW : wave_all;   // its number inside the group
     const int wm = wave / WN, wn = wave % WN;
+    // (the array itself when there is one group: a pointer variable in its place costs the
+    // 256-accumulator kernels registers, and they have none to spare)
+    decltype(auto) lds = [&]() -> decltype(auto) {
+        if constexpr (Cfg::KG == 1) return (lds_all);
+        else return lds_all + kg * Cfg::LDS_GROUP;
+    }();
 
     int tm, tn;
     tile_of_block<Cfg::GROUP>(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, tm, tn);
@@ -122,9 +140,11 @@ gemm_mfma16_kernel(const GemmArgs p) {
     // Split-K: this workgroup multiplies the K range [k0, k0 + K) of its tile; k_per_split is a
     // multiple of 128, so only the last piece can have a K tail.  Everything below works on
     // the local range.
-    const int k0 = SPLITK ? (int)blockIdx.y * p.k_per_split : 0;
+    // K groups: group g multiplies [g * K / KG, (g + 1) * K / KG); the launcher's caller makes
+    // sure K is a multiple of 128 * KG, so the groups run the same number of steps.
+    const int k0 = SPLITK ? (int)blockIdx.y * p.k_per_split : kg * (p.K / Cfg::KG);
     const int M = p.M, N = p.N;
-    const int K = SPLITK ? ((p.K - k0) < p.k_per_split ? (p.K - k0) : p.k_per_split) : p.K;
+    const int K = SPLITK ? ((p.K - k0) < p.k_per_split ? (p.K - k0) : p.k_per_split) : p.K / Cfg::KG;
     // K steps: an even number.  The aligned variant is only launched with K % 128 == 0; the
     // predicated one rounds up and the surplus (part of a) slab is zeroed in LDS.
     const int KT = EDGE ? ((K + 2 * BK - 1) / (2 * BK)) * 2 : K / BK;
@@ -426,6 +446,28 @@ gemm_mfma16_kernel(const GemmArgs p) {
     if constexpr (TRACE) {
         tr_store = tr_now();
         tr_loop = tr_store - tr_loop;
+    }
+    // ---- K groups: the second group's accumulators pass through its (drained) stages, 16
+    //      bytes per lane and tile, to the wave of the first group that owns the same sub-tile;
+    //      the sum is (first half of K) + (second half), a fixed order ----
+    if constexpr (Cfg::KG > 1) {
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");     // every wave is done with the last stage
+        f32x4_t* hand = (f32x4_t*)(lds_all + Cfg::LDS_GROUP) + (wave * (MI * NI)) * 64 + lane;
+        if (kg == 1) {
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int j = 0; j < NI; ++j) hand[(i * NI + j) * 64] = acc[i][j];
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        if (kg == 1) return;            // (waves that have ended no longer count at the barriers below)
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+            for (int j = 0; j < NI; ++j) {
+                const f32x4_t v = hand[(i * NI + j) * 64];
+                acc[i][j][0] += v[0]; acc[i][j][1] += v[1]; acc[i][j][2] += v[2]; acc[i][j][3] += v[3];
+            }
     }
     // ---- epilogue: C tile -> storage type -> per-wave LDS staging -> 16-byte row stores ----
     // acc[i][j][e] of lane l is C[m][n], m = i*16 + (l & 15), n = j*16 + 4*(l >> 4) + e
@@ -765,7 +807,10 @@ hipError_t launch_mfma16_kernel(const GemmArgs& args, hipStream_t stream) {
     const int grid = args.tiles_m * args.tiles_n;
     if (args.splits > 1) {
         if constexpr (TRACE) return hipErrorInvalidValue;   // no trace records from split-K launches
-        return launch_kernel(gemm_mfma16_kernel<Cfg, false, true>, dim3(grid, args.splits), dim3(Cfg::NT), stream, args);
+        if constexpr (Cfg::KG == 1)
+            return launch_kernel(gemm_mfma16_kernel<Cfg, false, true>, dim3(grid, args.splits), dim3(Cfg::NT), stream, args);
+        else
+            return hipErrorInvalidValue;        // K is already split inside the workgroup
     }
     return launch_kernel(gemm_mfma16_kernel<Cfg, TRACE>, dim3(grid), dim3(Cfg::NT), stream, args);
 }

@@ -89,7 +89,7 @@ int choose_tile_splits(const mi::KernelEntry& e, int M, int N, int K, bool split
                        int* k_per_split) {
     *k_per_split = K;
     static const int env = [] { const char* s = getenv("MI_GEMM_TILE_SPLITK"); return s ? atoi(s) : 0; }();
-    if (!splittable || e.kind != mi::KIND_MFMA16 || env == 1) return 1;
+    if (!splittable || e.kind != mi::KIND_MFMA16 || e.kg > 1 || env == 1) return 1;   // (K groups split K inside the workgroup)
     if (env > 1) {
         int s = env < K / 512 ? env : K / 512;
         if (s < 2 || (long long)((M + e.BM - 1) / e.BM) * ((N + e.BN - 1) / e.BN) * 256 * 256 * 4 >= 0x7fffffffLL) return 1;
@@ -414,6 +414,9 @@ int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const vo
         return MI_OK;
     }
 
+    if (e.kg > 1 && K % (128 * e.kg) != 0)
+        return fail(MI_ERR_UNSUPPORTED, "config %s splits K over %d groups of waves and needs K %% %d == 0", e.name,
+                    e.kg, 128 * e.kg);
     const bool edge = !shape_is_aligned(e, M, N, K, A, B, C);
     mi::LaunchFn fn = e.launch[dtype][edge ? 1 : 0];
     if (!fn) return fail(MI_ERR_UNSUPPORTED, "config %s has no %s kernel for dtype %d", e.name,
@@ -480,6 +483,7 @@ int mi_gemm_config_supports(int config, int dtype, int M, int N, int K) {
     if (is_split_k_decode(e.kind) || e.kind == mi::KIND_STREAM)
         return M <= e.BM && N % 4 == 0 && K % 64 == 0;
     if (e.kind == mi::KIND_WAVEK) return N % 4 == 0 && K % 64 == 0;
+    if (e.kg > 1 && K % (128 * e.kg) != 0) return 0;
     return e.launch[dtype][1] != nullptr;
 }
 

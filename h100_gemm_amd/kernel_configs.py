@@ -19,6 +19,8 @@ template takes (matmul_h100.cu.jinja:9-14) -- re-cast for CDNA4:
              tiles with K split over the waves of a workgroup, for outputs of few tiles with a
              long K, csrc/gemm_wavek_kernel.hpp)
     EPI      1: C tile transposed through LDS and written 16 bytes per lane, 0: 8-byte stores
+    KG       (mfma16, optional) 2: eight waves as two groups that each multiply half of K of the
+             same tile and add their accumulators through LDS (K % 256 == 0; tiles alone on a CU)
     DRAIN    (mfma16, optional) d > 0: a second barrier early in each K step (4*d MFMAs after the
              fragment reads) frees the current LDS stage, so the next loads are spread over most
              of the step instead of its second half
@@ -48,6 +50,8 @@ def config_name(c: dict) -> str:
             name += f"_b{c['DRAIN']}"
         if c.get("OCC", 1) != 1:
             name += f"_o{c['OCC']}"
+        if c.get("KG", 1) != 1:
+            name += f"_k{c['KG']}"
         return name
     if c["KIND"] == "ring16":
         return f"q{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_n{c['NS']}_g{c['GROUP']}"
@@ -65,7 +69,7 @@ def config_name(c: dict) -> str:
 
 
 def threads(c: dict) -> int:
-    return 256 if c["KIND"] in ("stream", "decode", "wavek") else c["WM"] * c["WN"] * 64
+    return 256 if c["KIND"] in ("stream", "decode", "wavek") else c["WM"] * c["WN"] * c.get("KG", 1) * 64
 
 
 def lds_bytes(c: dict) -> int:
@@ -77,7 +81,7 @@ def lds_bytes(c: dict) -> int:
         return c["NS"] * c["BN"] * 128
     if c["KIND"] == "wavek":     # per wave: the ring, or the padded fp32 partial tile if that is larger
         return 4 * max(c["NS"] * (c["BM"] + c["BN"]) * 128, c["BM"] * (c["BN"] + 4) * 4)
-    return 2 * (c["BM"] + c["BN"]) * 128
+    return c.get("KG", 1) * 2 * (c["BM"] + c["BN"]) * 128
 
 
 def is_valid_config(c: dict) -> bool:
@@ -111,7 +115,10 @@ def is_valid_config(c: dict) -> bool:
                 and c["BM"] * c["BN"] // 4 % 256 == 0
                 and (c["BM"] // 16) * (c["BN"] // 16) * 4 <= 256
                 and lds_bytes(c) * c.get("OCC", 1) <= 160 * 1024)
-    nt = c["WM"] * c["WN"] * 64
+    kg = c.get("KG", 1)
+    if kg not in (1, 2) or (kg == 2 and (c["KIND"] != "mfma16" or c["BM"] * c["BN"] * 4 > lds_bytes(c) // 2)):
+        return False            # the second K group's accumulators pass through its LDS stages
+    nt = c["WM"] * c["WN"] * kg * 64
     if nt > 1024 or nt < 64:
         return False
     if c["BM"] % (32 * c["WM"]) or c["BN"] % (32 * c["WN"]):
@@ -125,10 +132,10 @@ def is_valid_config(c: dict) -> bool:
     if c["KIND"] in ("mfma16", "ring16"):
         # 16x16x32 MFMA kernels: 4 accumulator registers per 16x16 tile; the two-stage kernel
         # runs with four or eight waves, the ring kernel with eight
-        if nt not in (256, 512) or c["BM"] * c["BN"] * 2 > lds_bytes(c):
+        if nt not in (256, 512) or c["BM"] * c["BN"] * 2 > lds_bytes(c) // kg:
             return False
         mi16, ni16 = 2 * mi, 2 * ni
-        rpp = nt // 8 if c["KIND"] == "mfma16" else nt // 4
+        rpp = nt // kg // 8 if c["KIND"] == "mfma16" else nt // 4
         if c["BM"] % rpp or c["BN"] % rpp:
             return False
         l = c["BM"] // rpp + c["BN"] // rpp
@@ -176,8 +183,10 @@ def _r(BM, BN, WM, WN, NS=4, GROUP=8):
     return dict(KIND="ring", BM=BM, BN=BN, WM=WM, WN=WN, NS=NS, GROUP=GROUP)
 
 
-def _m(BM, BN, WM, WN, GROUP=4, EFF=None, DRAIN=0, OCC=1, EFF_E=None):
+def _m(BM, BN, WM, WN, GROUP=4, EFF=None, DRAIN=0, OCC=1, EFF_E=None, KG=1):
     c = dict(KIND="mfma16", BM=BM, BN=BN, WM=WM, WN=WN, GROUP=GROUP)
+    if KG != 1:
+        c["KG"] = KG
     if EFF_E is not None:
         c["EFF_E"] = EFF_E
     if OCC != 1:
@@ -242,6 +251,7 @@ CONFIGS = [
     _m(256, 256, 2, 2, GROUP=8, DRAIN=1),
     _m(192, 192, 2, 2, DRAIN=1, EFF=0.80, EFF_E=0.91),
     _m(192, 128, 2, 2, DRAIN=1, EFF=0.74, EFF_E=0.85),
+    _m(128, 128, 2, 2, DRAIN=1, KG=2, EFF=0.51, EFF_E=0.74),
     _d(128, NS=3),
     _d(64, NS=4),
     _k(32, 32, NS=1, OCC=5, WK=(2.18, 0.0, 0.0775, 0.314)),

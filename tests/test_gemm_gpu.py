@@ -139,9 +139,17 @@ def test_c5_unaligned_full(mi, orc):
 
 # ------------------------------------------------------ every kernel configuration ----
 
-def all_configs(kinds=("tile", "ring", "mfma16", "ring16")):
+def all_configs(kinds=("tile", "ring", "mfma16", "ring16"), k_groups=True):
     from h100_gemm_amd import kernel_configs as kc
-    return [i for i, c in enumerate(kc.CONFIGS) if c["KIND"] in kinds]
+    return [i for i, c in enumerate(kc.CONFIGS) if c["KIND"] in kinds and (k_groups or c.get("KG", 1) == 1)]
+
+
+def k_for(config, K):
+    """K as the configuration can take it: a kernel that splits K over two groups of waves needs
+    equal halves of whole 128-deep double steps, so K is rounded up to a multiple of 256 for it"""
+    from h100_gemm_amd import kernel_configs as kc
+    kg = kc.CONFIGS[config].get("KG", 1) if config >= 0 else 1
+    return K if kg == 1 else -(-K // (128 * kg)) * 128 * kg
 
 
 @pytest.mark.parametrize("config", all_configs())
@@ -149,13 +157,13 @@ def test_every_config_bit_exact_on_integer_fill(mi, orc, config):
     # aligned (512^3: the aligned kernel), and ragged M, N, odd K (the predicated kernel)
     for M, N, K in [(512, 512, 512), (768, 1536, 1152), (257, 515, 77), (300, 200, 136), (65, 70, 33),
                     (256, 384, 191), (1, 1, 1)]:
-        check(mi, orc, M, N, K, "int", config=config, exact=True)
+        check(mi, orc, M, N, k_for(config, K), "int", config=config, exact=True)
 
 
 @pytest.mark.parametrize("config", all_configs())
 def test_every_config_uniform_within_tolerance(mi, orc, config):
     for M, N, K in [(1024, 768, 256), (255, 511, 129), (513, 391, 320)]:
-        check(mi, orc, M, N, K, "uniform", config=config)
+        check(mi, orc, M, N, k_for(config, K), "uniform", config=config)
 
 
 # ------------------------------------------------ decode (split-K streaming) kernels ----
@@ -207,6 +215,30 @@ def test_wave_split_k_kernels(mi, orc, config):
         with pytest.raises(mi.MiGemmError) as ei:
             Dev(mi, A, B, M, N).run(K, config=config)
         assert ei.value.code == mi._lib.MI_ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("config", [i for i in all_configs(("mfma16",)) if i not in all_configs(("mfma16",), k_groups=False)])
+def test_k_groups_inside_the_workgroup(mi, orc, config):
+    """Eight waves as two groups that each multiply half of K of the same tile and add their
+    accumulators through LDS: aligned and ragged M and N (the predicated variant), the shortest
+    K (one double step per group), fp16, epilogue, trace records; K that does not divide into
+    equal halves of whole double steps is refused."""
+    for M, N, K in [(512, 512, 256), (1536, 1536, 1536), (257, 515, 768), (1, 1, 256), (129, 127, 1280), (2048, 2048, 2048)]:
+        check(mi, orc, M, N, K, "int", config=config, exact=True)
+    check(mi, orc, 1024, 768, 2048, "uniform", config=config)
+    check(mi, orc, 300, 200, 512, "normal", config=config, dtype=orc.FP16)
+    check_epilogue(mi, orc, 384, 260, 1024, "int", -0.5, 2.75, config=config, exact=True)
+    check_epilogue(mi, orc, 200, 132, 512, "int", 2.0, -1.0, config=config, c_layout=mi.MI_C_COL_MAJOR, exact=True)
+    for K in (128, 384, 1000):
+        A, B = make_inputs(orc, 256, 256, K, "int")
+        with pytest.raises(mi.MiGemmError) as ei:
+            Dev(mi, A, B, 256, 256).run(K, config=config)
+        assert ei.value.code == mi._lib.MI_ERR_UNSUPPORTED
+    A, B = make_inputs(orc, 1536, 1536, 1536, "uniform")
+    d = Dev(mi, A, B, 1536, 1536)
+    C0 = d.run(1536, config=config)
+    for _ in range(3):
+        assert (d.run(1536, config=config) == C0).all()          # fixed summation order: bit-reproducible
 
 
 def test_wave_split_k_dispatch_and_determinism(mi, orc):
@@ -716,7 +748,8 @@ def test_db_trace_records(mi, orc):
     rec = records(mi.MI_CONFIG_AUTO)
     tiled = [i for i, c in enumerate(kc.CONFIGS) if c["KIND"] == "mfma16" and c.get("EFF")]
     assert len(rec) in {-(-M // kc.CONFIGS[i]["BM"]) * -(-N // kc.CONFIGS[i]["BN"]) for i in tiled}
-    assert (rec[:, 3] == K // 64).all()
+    # K steps per workgroup (per group of waves where a kernel splits K over two of them)
+    assert (rec[:, 3] == K // 64).all() or (rec[:, 3] == K // 128).all()
     # asked for by name, the small-tile kernel runs and leaves the buffer untouched
     assert len(records(mi.select_config(M, N, K))) == 0
 
@@ -843,7 +876,7 @@ def test_alpha_beta_every_tiled_config_bit_exact_on_integer_fill(mi, orc, config
     for (M, N, K), (alpha, beta) in [((512, 512, 512), (0.5, 3.0)), ((257, 515, 77), (-2.0, 0.25)),
                                      ((300, 200, 136), (3.0, -1.5)), ((256, 384, 191), (1.0, 7.0)),
                                      ((512, 768, 256), (0.25, 0.0))]:
-        check_epilogue(mi, orc, M, N, K, "int", alpha, beta, config=config, exact=True)
+        check_epilogue(mi, orc, M, N, k_for(config, K), "int", alpha, beta, config=config, exact=True)
 
 
 @pytest.mark.parametrize("config", all_configs(("stream", "decode")))
@@ -895,7 +928,7 @@ def test_epilogue_fp16_and_argument_errors(mi, orc):
 
 # ------------------------------------------- split-K of the tiled 16x16x32 kernel ----------
 
-@pytest.mark.parametrize("config", all_configs(("mfma16",)))
+@pytest.mark.parametrize("config", all_configs(("mfma16",), k_groups=False))
 def test_tiled_split_k_bit_exact_on_integer_fill(mi, orc, config):
     """Few tiles and a long K: the K range is cut into pieces, fp32 partials are added in order.
     Integer fills keep every partial sum exact, so the result must match the oracle's bits."""
@@ -935,7 +968,7 @@ def test_tiled_split_k_random_shapes_and_alignments(mi, orc):
     # candidate tile of it
     from h100_gemm_amd import kernel_configs as kc
     rng = np.random.default_rng(20241125)
-    configs = [-1] + [i for i, c in enumerate(kc.CONFIGS) if c["KIND"] == "mfma16" and c.get("EFF")]
+    configs = [-1] + [i for i, c in enumerate(kc.CONFIGS) if c["KIND"] == "mfma16" and c.get("EFF") and c.get("KG", 1) == 1]
     for it in range(32):
         M = int(rng.integers(1, 420))
         N = int(rng.integers(1, 110)) * 4

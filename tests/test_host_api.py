@@ -144,6 +144,12 @@ def test_config_table(mi):
             assert L.mi_gemm_config_supports(i, 0, 1000, 780, 4100) == 0
             assert L.mi_gemm_config_supports(i, 0, 1000, 778, 4096) == 0
             assert mi.config_grid(i, 1000, 780, 4100) == 0
+        elif c.get("KG", 1) > 1:
+            # K split over groups of waves inside the workgroup: any M, N; K in equal halves of whole double steps
+            assert L.mi_gemm_config_supports(i, 0, 4095, 6143, 3072) == 1
+            assert L.mi_gemm_config_supports(i, 0, 4095, 6143, 3073) == 0
+            assert L.mi_gemm_config_supports(i, 0, 512, 512, 384) == 0
+            assert mi.config_grid(i, 1000, 777, 256) == -(-1000 // c["BM"]) * -(-777 // c["BN"])
         else:
             tiles = -(-1000 // c["BM"]) * -(-777 // c["BN"])
             assert mi.config_grid(i, 1000, 777, 64) == tiles
