@@ -45,6 +45,9 @@ WORKLOADS = {
     # outputs of few tiles (not BASELINE configurations; for the profiles of the small-tile kernel)
     "fewtile512": (512, 512, 4096, "uniform"),
     "fewtile1024": (1024, 1024, 4096, "uniform"),
+    # 144 and 256 tiles of 128x128: one workgroup per CU at most (the kernel with two K groups)
+    "square1536": (1536, 1536, 1536, "uniform"),
+    "square2048": (2048, 2048, 2048, "uniform"),
 }
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (the summaries under
 # profiles/ give the commands), scaled by the same counters on a copy kernel of known size:
