@@ -251,7 +251,7 @@ CONFIGS = [
     _m(256, 256, 2, 2, GROUP=8, DRAIN=1),
     _m(192, 192, 2, 2, DRAIN=1, EFF=0.80, EFF_E=0.91),
     _m(192, 128, 2, 2, DRAIN=1, EFF=0.74, EFF_E=0.85),
-    _m(128, 128, 2, 2, DRAIN=1, KG=2, EFF=0.51, EFF_E=0.74),
+    _m(128, 128, 2, 2, DRAIN=1, KG=2, EFF=0.51, EFF_E=0.93),
     _d(128, NS=3),
     _d(64, NS=4),
     _k(32, 32, NS=1, OCC=5, WK=(2.18, 0.0, 0.0775, 0.314)),
