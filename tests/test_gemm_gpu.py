@@ -239,6 +239,15 @@ def test_k_groups_inside_the_workgroup(mi, orc, config):
     C0 = d.run(1536, config=config)
     for _ in range(3):
         assert (d.run(1536, config=config) == C0).all()          # fixed summation order: bit-reproducible
+    # seeded sweep: ragged M and N, base pointers at arbitrary even byte offsets (the predicated variant)
+    rng = np.random.default_rng(20241126)
+    for it in range(12):
+        M, N, K = int(rng.integers(1, 600)), int(rng.integers(1, 600)), 256 * int(rng.integers(1, 6))
+        offA, offB, offC = (int(2 * rng.integers(0, 16)) for _ in range(3))
+        print(f"case {it}: M={M} N={N} K={K} offsets {offA},{offB},{offC}", flush=True)
+        C, ref, guard = _run_offset(mi, orc, config, M, N, K, offA, offB, offC)
+        assert (C == ref).all(), f"{int((C != ref).sum())} elements differ"
+        assert (guard == 0xEEEE).all(), "bytes outside C were written"
 
 
 def test_wave_split_k_dispatch_and_determinism(mi, orc):
