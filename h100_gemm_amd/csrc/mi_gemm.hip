@@ -238,6 +238,13 @@ bool shape_is_aligned(const mi::KernelEntry& e, int M, int N, int K, const void*
            aligned16(C);
 }
 
+// Shapes a launch accepts: positive extents, `int` element indices as in the reference
+// (reference.h:30,40 index with int) and 32-bit byte offsets inside one tile's row panel.
+bool shape_in_range(int M, int N, int K) {
+    return M > 0 && N > 0 && K > 0 && (long long)M * K <= 0x7fffffffLL && (long long)N * K <= 0x7fffffffLL &&
+           (long long)M * N <= 0x7fffffffLL && (long long)K * 2 * 256 <= 0x7fffffffLL;
+}
+
 int check_args(int config, int dtype, int M, int N, int K, const void* A, const void* B,
                const void* C) {
     if (dtype != MI_DTYPE_BF16 && dtype != MI_DTYPE_FP16)
@@ -478,7 +485,7 @@ int mi_gemm_config_lds_bytes(int config) {
 int mi_gemm_config_supports(int config, int dtype, int M, int N, int K) {
     if (config < 0 || config >= mi::kNumKernels) return 0;
     if (dtype != MI_DTYPE_BF16 && dtype != MI_DTYPE_FP16) return 0;
-    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    if (!shape_in_range(M, N, K)) return 0;
     const mi::KernelEntry& e = mi::kKernels[config];
     if (is_split_k_decode(e.kind) || e.kind == mi::KIND_STREAM)
         return M <= e.BM && N % 4 == 0 && K % 64 == 0;
@@ -488,7 +495,7 @@ int mi_gemm_config_supports(int config, int dtype, int M, int N, int K) {
 }
 
 int mi_gemm_config_grid(int config, int M, int N, int K) {
-    if (config < 0 || config >= mi::kNumKernels || M <= 0 || N <= 0 || K <= 0) return 0;
+    if (config < 0 || config >= mi::kNumKernels || !shape_in_range(M, N, K)) return 0;
     const mi::KernelEntry& e = mi::kKernels[config];
     if (e.kind == mi::KIND_STREAM) return M > e.BM || K % 64 != 0 ? 0 : (N + e.BN - 1) / e.BN;
     if (is_split_k_decode(e.kind)) {
@@ -507,6 +514,7 @@ int mi_gemm_config_grid(int config, int M, int N, int K) {
 
 int mi_gemm_select_config(int dtype, int M, int N, int K) {
     (void)dtype;
+    if (!shape_in_range(M, N, K)) return -1;
     // pointer alignment is unknown here: assume the usual 256-byte aligned allocations
     const bool streamable = N % 4 == 0 && K % 64 == 0;
     const int tuned = tuned_config(M, N, K, streamable);
@@ -551,9 +559,8 @@ int mi_gemm_bf16(int M, int N, int K, const uint16_t* A, const uint16_t* B, uint
 
 size_t mi_gemm_workspace_bytes(int config, int dtype, int M, int N, int K, int c_layout) {
     if (dtype != MI_DTYPE_BF16 && dtype != MI_DTYPE_FP16) return 0;
-    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    if (!shape_in_range(M, N, K)) return 0;
     if (config != MI_CONFIG_AUTO && (config < 0 || config >= mi::kNumKernels)) return 0;
-    if ((long long)M * N > 0x7fffffffLL) return 0;
     if (c_layout == MI_C_COL_MAJOR) {
         const int t = M;
         M = N;

@@ -128,7 +128,8 @@ int mi_gemm_num_configs(void);
 const char* mi_gemm_config_name(int config);
 /* Index of the config with that name, or -1. */
 int mi_gemm_find_config(const char* name);
-/* The config MI_CONFIG_AUTO resolves to for this shape (never negative for valid shapes). */
+/* The config MI_CONFIG_AUTO resolves to for this shape; -1 for a shape no launch accepts
+ * (an extent <= 0, or a matrix of more than 2^31-1 elements). */
 int mi_gemm_select_config(int dtype, int M, int N, int K);
 /* Number of `M N K config-name` lines loaded from the file named by the environment variable
  * MI_GEMM_TUNED_FILE (read once, on first use; 0 without it).  MI_CONFIG_AUTO takes a listed

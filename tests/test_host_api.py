@@ -103,6 +103,14 @@ def test_argument_validation_needs_no_device(mi):
     assert L.mi_gemm_epilogue(-1, bf, 8, 8, 8, 1, 1, 1, float("nan"), 0.0, 0, None) == mi._lib.MI_ERR_INVALID
     assert L.mi_gemm_epilogue(-1, bf, 8, 0, 8, 1, 1, 1, 1.0, 0.0, mi.MI_C_COL_MAJOR, None) == mi._lib.MI_ERR_INVALID
     assert L.mi_gemm_epilogue(-1, bf, 8, 8, 8, 1, None, 1, 1.0, 0.0, mi.MI_C_COL_MAJOR, None) == mi._lib.MI_ERR_INVALID
+    # the shape queries apply the same limits instead of computing with extents a launch refuses
+    big = 2**31 - 1
+    for M, N, K in [(big, big, big), (0, 8, 8), (8, -1, 8), (70000, 70000, 8), (1, 1, 4194304)]:
+        assert L.mi_gemm_select_config(bf, M, N, K) == -1
+        assert L.mi_gemm_config_supports(0, bf, M, N, K) == 0
+        assert L.mi_gemm_config_grid(0, M, N, K) == 0
+        assert L.mi_gemm_workspace_bytes(-1, bf, M, N, K, 0) == 0
+        assert L.mi_gemm_trace_words(M, N, K) == 1
     with pytest.raises(mi.MiGemmError):
         mi.runKernel(8, 8, 0, 1, 1, 1)
     with pytest.raises(ValueError):
@@ -371,6 +379,9 @@ def test_automatic_choice_always_names_a_kernel_that_can_run_the_shape(mi):
             M, N, K = rng.choice([1, 3, 100000]), rng.choice([1, 4, 8, 200000]), rng.choice([1, 64, 4096, 100000])
         M, N, K = int(M), int(N), int(K)
         c = mi.select_config(M, N, K)
+        if max(M * K, N * K, M * N) > 2**31 - 1:          # a shape no launch accepts
+            assert c == -1, (M, N, K, c)
+            continue
         assert 0 <= c < mi.num_configs(), (M, N, K, c)
         assert L.mi_gemm_config_supports(c, 0, M, N, K) == 1, (M, N, K, mi.config_name(c))
         assert mi.config_grid(c, M, N, K) > 0, (M, N, K, mi.config_name(c))
