@@ -46,6 +46,8 @@ WORKLOADS = {
     "fewtile512": (512, 512, 4096, "uniform"),
     "fewtile1024": (1024, 1024, 4096, "uniform"),
     # 144 and 256 tiles of 128x128: one workgroup per CU at most (the kernel with two K groups)
+    # 225 tiles of 96x96, one per CU at most, K too short to split over the waves (the shared-ring kernel)
+    "mid1440": (1440, 1440, 1472, "uniform"),
     "square1536": (1536, 1536, 1536, "uniform"),
     "square2048": (2048, 2048, 2048, "uniform"),
 }

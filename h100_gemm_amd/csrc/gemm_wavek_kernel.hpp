@@ -1,7 +1,8 @@
-// gemm_wavek_kernel.hpp -- gfx950 GEMM kernel for outputs of few tiles with a long K:
+// gemm_wavek_kernel.hpp -- gfx950 GEMM kernels for outputs of few tiles:
 //
-//   C[M,N] = A[M,K] . B[N,K]^T     small tiles, K split over the four waves of a workgroup,
-//                                  one kernel, no workspace
+//   C[M,N] = A[M,K] . B[N,K]^T     small tiles, one kernel, no workspace
+//   gemm_wavek_kernel:        K split over the four waves of a workgroup (few tiles, long K)
+//   gemm_shared_ring_kernel:  2 x 2 waves over the tile, one shared ring (further down)
 //
 // A 512 x 512 or 1024 x 1024 output has 16 or 64 tiles of 128 x 128: most of the chip idles,
 // or K is cut into pieces whose partial sums make a round trip through memory and a second
@@ -213,6 +214,195 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
             *(u32x2_t*)((unsigned char*)p.C + ((size_t)(row0 + m) * p.ldc + col0 + n) * 2) = w2;
         }
     }
+}
+
+// ---------------------------------------------------------------------------------------
+// Shared-ring variant, for outputs whose tiles of BM x BN number at most one per CU but are too
+// large to be multiplied whole by every wave (96 x 96: 1536^2 is 256 of them, where 128 x 128
+// tiles leave 112 CUs idle and each busy CU takes in a third more).  The four waves form a
+// 2 x 2 grid over the tile and walk all of K together; one ring of NS stages, each one
+// 64-deep unit of (BM + BN) rows laid out as above, is filled by all four waves (a quarter of
+// a stage's load instructions each) and read by all four.  One barrier per unit: it tells
+// every wave that the unit it is about to read has landed (each wave has waited for its own
+// loads) and that the stage of the unit before it has been read by everyone, so that the
+// request NS - 1 units ahead can take that stage.  The workgroup is bound by the same intake
+// of a CU as the kernel above; the deeper ring keeps NS - 1 units in flight while one is
+// multiplied.  Same preconditions, same stage layout, same fragment reads.
+template <int BM_, int BN_, int NS_, int DT_>
+struct SharedRingConfig {
+    static constexpr int BM = BM_, BN = BN_, NS = NS_, DT = DT_;
+    static constexpr int NT = 256, NW = 4;
+    static constexpr int TM = BM / 2, TN = BN / 2;           // wave tile of the 2 x 2 wave grid
+    static constexpr int MI = TM / 16, NI = TN / 16;
+    static constexpr int L = (BM + BN) / 8;                  // load instructions per unit
+    static constexpr int LW = L / NW;                        // ... of one wave
+    static constexpr int STAGE = (BM + BN) * 128;
+    static constexpr int RING = NS * STAGE;
+    static constexpr int PITCH = BN + 4;                     // floats per row of the staged C tile (bank spread)
+    static constexpr int PART = BM * PITCH * 4;
+    static constexpr int LDS_BYTES = RING > PART ? RING : PART;
+    static constexpr int QUADS = BM * BN / 4 / NT;           // 4-element groups of C per thread
+    static_assert(BM % 32 == 0 && BN % 32 == 0, "wave tiles of whole 16x16 MFMA tiles");
+    static_assert(L % NW == 0, "a stage's load instructions divide over the waves");
+    static_assert(NS >= 3 && (NS - 1) * LW <= 63, "a unit being read, one being multiplied, the rest in flight; vmcnt is a 6-bit counter");
+    static_assert(BM * BN / 4 % NT == 0, "the C tile divides over the threads");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
+};
+
+template <class Cfg>
+__global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs p) {
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::NS, DT = Cfg::DT;
+    constexpr int MI = Cfg::MI, NI = Cfg::NI, LW = Cfg::LW, STAGE = Cfg::STAGE;
+    constexpr int TM = Cfg::TM, TN = Cfg::TN, PITCH = Cfg::PITCH;
+
+    __shared__ __attribute__((aligned(128))) unsigned char lds[Cfg::LDS_BYTES];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int M = p.M, N = p.N, K = p.K;
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    int tm, tn;
+    tile_of_block<4>(blockIdx.x, gridDim.x, tiles_m, tiles_n, tm, tn);
+    const int row0 = tm * BM, col0 = tn * BN;
+    const int KT = K / 64;                                   // units of K
+
+    const int rowsA = (M - row0) < BM ? (M - row0) : BM;
+    const int rowsB = (N - col0) < BN ? (N - col0) : BN;
+    const unsigned char* Ab = (const unsigned char*)p.A + (size_t)row0 * p.lda * 2;
+    const unsigned char* Bb = (const unsigned char*)p.B + (size_t)col0 * p.ldb * 2;
+    const uint32_t bytesA = (uint32_t)((rowsA - 1) * p.lda + K) * 2u;
+    const uint32_t bytesB = (uint32_t)((rowsB - 1) * p.ldb + K) * 2u;
+    const __amdgpu_buffer_rsrc_t rsrcA = __builtin_amdgcn_make_buffer_rsrc((void*)Ab, 0, (int)bytesA, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrcB = __builtin_amdgcn_make_buffer_rsrc((void*)Bb, 0, (int)bytesB, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrcNone = __builtin_amdgcn_make_buffer_rsrc((void*)Ab, 0, 0, 0x00020000);
+
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
+    auto dma = [&](const __amdgpu_buffer_rsrc_t& rsrc, uint32_t voff, uint32_t dst) __attribute__((always_inline)) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                     :: "s"(dst), "v"(voff), "s"(rsrc) : "memory");
+    };
+    auto swz = [](int row) __attribute__((always_inline)) { return (row >> 1) & 7; };
+    // load instruction wave * LW + q of a unit fills stage rows 8 * that .. + 7 (A rows first,
+    // then B rows): this lane's byte offset inside A or B, k offset added per request
+    const int lr = lane >> 3, lc = lane & 7;
+    uint32_t voff[LW];
+#pragma unroll
+    for (int q = 0; q < LW; ++q) {
+        const int row = (wave * LW + q) * 8 + lr;
+        const int chunk = lc ^ swz(row);
+        voff[q] = row < BM ? (uint32_t)(row * p.lda + chunk * 8) * 2u
+                           : (uint32_t)((row - BM) * p.ldb + chunk * 8) * 2u;
+    }
+    // `rq_unit` follows the unit about to be requested; requests past the last unit fetch nothing
+    int rq_unit = 0;
+    auto request = [&](int stage) __attribute__((always_inline)) {
+        const bool live = rq_unit < KT;
+        const uint32_t kb = (uint32_t)rq_unit * 128u;
+        ++rq_unit;
+        const uint32_t dst = lds_base + (uint32_t)(stage * STAGE + wave * LW * 1024);
+#pragma unroll
+        for (int q = 0; q < LW; ++q)
+            dma(live ? ((wave * LW + q) * 8 < BM ? rsrcA : rsrcB) : rsrcNone, voff[q] + kb, dst + (uint32_t)(q * 1024));
+    };
+
+    // fragment read: lane holds row l & 15 of a 16-row block, chunk 4*slice + (l >> 4)
+    const int l16 = lane & 15, q4 = lane >> 4;
+    int rd_off[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) rd_off[ks] = l16 * 128 + ((((ks << 2) | q4) ^ swz(l16)) << 4);
+    const int a_wave = wm * TM * 128, b_wave = (BM + wn * TN) * 128;
+
+    f32x4_t acc[MI][NI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) acc[i][j] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+#pragma unroll
+    for (int i = 0; i < NS - 1; ++i) request(i);
+
+    // The fragments of unit u + 1 are read while unit u is multiplied (one wave per SIMD has
+    // nothing else to hide the LDS latency behind), so a unit must have landed one step before
+    // it is multiplied: NS - 2 units are in flight while one is read and one multiplied.
+    // Two register sets, used in turn (a copy from "next" to "current" at the end of a step
+    // lets the compiler move the reads behind the MFMAs again).
+    u32x4_t fa[2][2][MI], fb[2][2][NI];                      // [set][slice][block]
+    auto read_unit = [&](int stage, u32x4_t (&a)[2][MI], u32x4_t (&b)[2][NI]) __attribute__((always_inline)) {
+        const unsigned char* st = lds + stage * STAGE;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+            for (int i = 0; i < MI; ++i) a[ks][i] = *(const u32x4_t*)(st + a_wave + i * 2048 + rd_off[ks]);
+#pragma unroll
+            for (int j = 0; j < NI; ++j) b[ks][j] = *(const u32x4_t*)(st + b_wave + j * 2048 + rd_off[ks]);
+        }
+    };
+    int s = 0;                                               // stage of the unit being multiplied
+    // one step: unit u (fragments in set CUR) is multiplied while unit u + 1 is read into the other set
+    auto step = [&](auto cur_c) __attribute__((always_inline)) {
+        constexpr int CUR = decltype(cur_c)::value;
+        // this wave's loads of unit u + 1 have landed; after the barrier everyone's have, and
+        // everyone has multiplied unit u - 1, whose stage takes the request NS - 1 units ahead
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"((NS - 3) * LW) : "memory");
+        request(s == 0 ? NS - 1 : s - 1);
+        read_unit(s + 1 == NS ? 0 : s + 1, fa[CUR ^ 1], fb[CUR ^ 1]);   // (past the last unit: zeros or stale rows, never multiplied)
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int j = 0; j < NI; ++j)
+                    acc[i][j] = mfma_16x16x32<DT>(fb[CUR][ks][j], fa[CUR][ks][i], acc[i][j]);
+        __builtin_amdgcn_sched_barrier(0);
+        s = s + 1 == NS ? 0 : s + 1;
+    };
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"((NS - 2) * LW) : "memory");     // unit 0 has landed
+    read_unit(0, fa[0], fb[0]);
+    int u = 0;
+    for (; u + 2 <= KT; u += 2) {
+        step(std::integral_constant<int, 0>{});
+        step(std::integral_constant<int, 1>{});
+    }
+    if (u < KT) step(std::integral_constant<int, 0>{});
+    // requests past the last unit (empty descriptor: zeros) are still heading for the ring, and
+    // other waves may still be reading the last stage: drain and meet before C takes its place
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+
+    // ---- the C tile through LDS as fp32, then scaled, rounded once and stored 8 bytes per lane ----
+    // acc[i][j][e] of lane l is C[m][n], m = wm*TM + i*16 + (l & 15), n = wn*TN + j*16 + 4*(l >> 4) + e
+    float* part = (float*)lds;
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+            *(f32x4_t*)(part + (wm * TM + i * 16 + l16) * PITCH + wn * TN + j * 16 + 4 * q4) = acc[i][j];
+    __syncthreads();
+    const bool scaled = p.alpha != 1.0f || p.beta != 0.0f;
+#pragma unroll
+    for (int it = 0; it < Cfg::QUADS; ++it) {
+        const int q = it * 256 + tid;
+        const int m = q / (BN / 4), n = (q % (BN / 4)) * 4;
+        f32x4_t sum = *(const f32x4_t*)(part + m * PITCH + n);
+        if (scaled) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sum[e] = mul_add_unfused(sum[e], p.alpha, p.beta);
+        }
+        if (row0 + m < M && col0 + n < N) {                  // N % 4 == 0 is a launch precondition
+            u32x2_t w2;
+            w2[0] = cvt_store2<DT>(sum[0], sum[1]);
+            w2[1] = cvt_store2<DT>(sum[2], sum[3]);
+            *(u32x2_t*)((unsigned char*)p.C + ((size_t)(row0 + m) * p.ldc + col0 + n) * 2) = w2;
+        }
+    }
+}
+
+template <class Cfg>
+hipError_t launch_shared_ring_kernel(const DecodeArgs& a, hipStream_t stream) {
+    const int tiles = ((a.M + Cfg::BM - 1) / Cfg::BM) * ((a.N + Cfg::BN - 1) / Cfg::BN);
+    return launch_kernel(gemm_shared_ring_kernel<Cfg>, dim3(tiles), dim3(256), stream, a);
 }
 
 template <class Cfg>

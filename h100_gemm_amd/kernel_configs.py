@@ -28,11 +28,15 @@ template takes (matmul_h100.cu.jinja:9-14) -- re-cast for CDNA4:
              register-staged predicated kernel runs best with eight waves)
     EFF      (optional) per-CU throughput relative to the 256x256 tile, measured at 8192^3;
              configs that carry it are the candidates of the automatic shape -> kernel choice
+    SHARED   (wavek, optional) 1: the four waves form a 2 x 2 grid over the tile and share one
+             ring of NS stages (a barrier per 64-deep unit, no partial tiles to add) instead of
+             each multiplying the whole tile over a quarter of K -- for outputs of up to a few
+             tiles per CU with a K too short to split four ways, or tiles too large for that
     WK       (wavek, optional) time model in microseconds, (fixed, per round, per unit, per
              tile): fixed + rounds of co-resident workgroups (tiles / (CUs x OCC), rounded up)
              x per round + tiles per CU (rounded up) x (per tile + K/64 x per unit);
-             non-negative least squares on 89 shapes; configs that carry it join the
-             automatic choice
+             non-negative least squares on 89 shapes (the 96x64 shared-ring config: x 1.07, its
+             fit being the loosest); configs that carry it join the automatic choice
     EFF_E    (optional) throughput of the predicated variant relative to the aligned one, from
              7000^3, 6000^3 and 5000^3 (default 0.85); used for shapes the aligned variant cannot run
 
@@ -60,7 +64,7 @@ def config_name(c: dict) -> str:
     if c["KIND"] == "decode":
         return f"d{c['BM']}x{c['BN']}_n{c['NS']}"
     if c["KIND"] == "wavek":
-        return f"k{c['BM']}x{c['BN']}_n{c['NS']}"
+        return f"k{c['BM']}x{c['BN']}_{'s' if c.get('SHARED') else 'n'}{c['NS']}"
     name = (f"t{c['BM']}x{c['BN']}_w{c['WM']}x{c['WN']}_s{c['SWZ']}_g{c['GROUP']}"
             f"_o{c['OCC']}_d{c['DTL']}_e{c['EPI']}")
     if (c.get("EWM", c["WM"]), c.get("EWN", c["WN"])) != (c["WM"], c["WN"]):
@@ -79,6 +83,8 @@ def lds_bytes(c: dict) -> int:
         return 4 * c["NS"] * (c["BM"] + c["BN"]) * 128
     if c["KIND"] == "decode":
         return c["NS"] * c["BN"] * 128
+    if c["KIND"] == "wavek" and c.get("SHARED"):     # one ring for the workgroup, or the padded fp32 C tile
+        return max(c["NS"] * (c["BM"] + c["BN"]) * 128, c["BM"] * (c["BN"] + 4) * 4)
     if c["KIND"] == "wavek":     # per wave: the ring, or the padded fp32 partial tile if that is larger
         return 4 * max(c["NS"] * (c["BM"] + c["BN"]) * 128, c["BM"] * (c["BN"] + 4) * 4)
     return c.get("KG", 1) * 2 * (c["BM"] + c["BN"]) * 128
@@ -108,6 +114,12 @@ def is_valid_config(c: dict) -> bool:
         return (c["BM"] in (64, 128) and c["BN"] % 32 == 0 and c["NS"] >= 3
                 and (c["NS"] - 1) * (c["BM"] // 32 + c["BN"] // 32) <= 63
                 and lds_bytes(c) <= 160 * 1024)
+    if c["KIND"] == "wavek" and c.get("SHARED"):
+        # 2 x 2 waves over the tile, one ring: per wave and stage (BM + BN) / 32 loads, NS - 1 stages outstanding
+        return (c["BM"] % 32 == 0 and c["BN"] % 32 == 0 and c["NS"] >= 3
+                and (c["NS"] - 1) * ((c["BM"] + c["BN"]) // 32) <= 63
+                and c["BM"] * c["BN"] // 4 % 256 == 0
+                and lds_bytes(c) * c.get("OCC", 1) <= 160 * 1024)
     if c["KIND"] == "wavek":
         # per wave and ring stage (BM + BN) / 8 direct-to-LDS loads, NS stages outstanding
         return (c["BM"] % 16 == 0 and c["BN"] % 16 == 0 and c["NS"] >= 1
@@ -206,8 +218,10 @@ def _s(BM, NS):
     return dict(KIND="stream", BM=BM, BN=32, NS=NS)
 
 
-def _k(BM, BN, NS, WK=None, OCC=1):
+def _k(BM, BN, NS, WK=None, OCC=1, SHARED=0):
     c = dict(KIND="wavek", BM=BM, BN=BN, NS=NS)
+    if SHARED:
+        c["SHARED"] = 1         # 2 x 2 waves over the tile and one ring, instead of K split over the waves
     if OCC != 1:
         c["OCC"] = OCC          # workgroups that fit a CU together (LDS): rounds of the time model
     if WK is not None:
@@ -251,7 +265,7 @@ CONFIGS = [
     _m(256, 256, 2, 2, GROUP=8, DRAIN=1),
     _m(192, 192, 2, 2, DRAIN=1, EFF=0.80, EFF_E=0.91),
     _m(192, 128, 2, 2, DRAIN=1, EFF=0.74, EFF_E=0.85),
-    _m(128, 128, 2, 2, DRAIN=1, KG=2, EFF=0.51, EFF_E=0.93),
+    _m(128, 128, 2, 2, DRAIN=1, KG=2, EFF=0.64, EFF_E=0.93),
     _d(128, NS=3),
     _d(64, NS=4),
     _k(32, 32, NS=1, OCC=5, WK=(2.18, 0.0, 0.0775, 0.314)),
@@ -260,6 +274,10 @@ CONFIGS = [
     _k(64, 64, NS=1, OCC=2, WK=(1.93, 2.19, 0.1792, 0.0)),
     _k(64, 64, NS=2, WK=(0.88, 2.81, 0.1648, 0.0)),
     _k(96, 64, NS=2, WK=(1.35, 4.06, 0.2306, 0.0)),
+    _k(96, 96, NS=4, SHARED=1, WK=(1.23, 2.555, 0.3643, 0.0)),
+    _k(64, 64, NS=4, SHARED=1, OCC=2, WK=(1.94, 1.270, 0.1847, 0.0)),
+    _k(96, 64, NS=4, SHARED=1, OCC=2, WK=(2.58, 1.43, 0.2584, 0.0)),
+    _k(64, 32, NS=4, SHARED=1, OCC=3, WK=(1.99, 0.958, 0.1252, 0.0)),
 ]
 
 assert all(is_valid_config(c) for c in CONFIGS), [config_name(c) for c in CONFIGS if not is_valid_config(c)]

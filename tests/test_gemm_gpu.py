@@ -257,6 +257,16 @@ def test_wave_split_k_dispatch_and_determinism(mi, orc):
     for M, N, K in [(512, 512, 4096), (1024, 1024, 4096), (512, 512, 4100), (512, 510, 4096), (640, 384, 3328)]:
         check(mi, orc, M, N, K, "int", exact=True)
     assert kc.CONFIGS[mi.select_config(512, 512, 4096)]["KIND"] == "wavek"
+    # the shared-ring kernels through the automatic choice (also a K that is no multiple of 64:
+    # the tiled kernels give the same answers)
+    for M, N, K in [(1440, 1440, 1472), (1344, 1344, 1344), (1536, 1472, 320), (1440, 1440, 1480)]:
+        check(mi, orc, M, N, K, "int", exact=True)
+    assert kc.CONFIGS[mi.select_config(1440, 1440, 1472)].get("SHARED") == 1
+    A, B = make_inputs(orc, 1440, 1440, 1472, "uniform")
+    d = Dev(mi, A, B, 1440, 1440)
+    C0 = d.run(1472)
+    for _ in range(3):
+        assert (d.run(1472) == C0).all()
     A, B = make_inputs(orc, 1024, 1024, 4096, "uniform")
     d = Dev(mi, A, B, 1024, 1024)
     C0 = d.run(4096)

@@ -182,6 +182,13 @@ def test_config_table(mi):
     assert kc.CONFIGS[mi.select_config(1024, 1024, 4096)]["KIND"] == "wavek"
     assert kc.CONFIGS[mi.select_config(512, 512, 4100)]["KIND"] == "mfma16"
     assert kc.CONFIGS[mi.select_config(512, 510, 4096)]["KIND"] == "mfma16"
+    # a mid-sized output with a K of moderate length: small tiles on a shared ring (K is not split
+    # over the waves), also with a short K and many tiles, where the K-splitting ones are shut out
+    assert not kc.CONFIGS[mi.select_config(512, 512, 4096)].get("SHARED")
+    for M, N, K in [(1440, 1440, 1472), (1344, 1344, 1344), (1536, 1472, 320)]:
+        c = kc.CONFIGS[mi.select_config(M, N, K)]
+        assert c["KIND"] == "wavek" and c.get("SHARED") == 1, (M, N, K, c)
+    assert mi.config_name(mi.select_config(1536, 1536, 1536)) == "m128x128_w2x2_g4_b1_k2"
     # wave quantisation: 256 CUs; 8192^2 fills four rounds of 256x256 tiles, 4095x6143 fills
     # two rounds of 256x192 tiles exactly (256x256 would leave half of the second round
     # idle), and 512^2 is a single partial round whatever the tiled kernel: the small-tile
