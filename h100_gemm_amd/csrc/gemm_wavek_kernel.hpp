@@ -43,8 +43,9 @@
 // single stage and one workgroup per CU only, were far behind the tiled kernels (2048^3:
 // 26.5 us against 19.6): alone and with one stage, loading and multiplying take turns.
 // Rows of A past M and rows of B past N are never fetched (the buffer descriptors end at the
-// last valid row of the tile).  Preconditions, checked by the launcher's caller: K % 64 == 0,
-// N % 4 == 0, 16-byte aligned A and B rows, 8-byte aligned C.
+// last valid row of the tile).  Preconditions, checked by the launcher's caller: K % 8 == 0 and
+// 16-byte aligned A and B (rows that start on 16-byte boundaries; a partial last unit of K is
+// filled up with zeros), N % 4 == 0, 8-byte aligned C.
 // The reference has no counterpart: its kernels use one tile size (matmul_utils.cuh:362).
 #pragma once
 
@@ -92,7 +93,8 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
     int tm, tn;
     tile_of_block<4>(blockIdx.x, gridDim.x, tiles_m, tiles_n, tm, tn);
     const int row0 = tm * BM, col0 = tn * BN;
-    const int KT = K / 64;                                   // units of K
+    const int KT = (K + 63) / 64;                            // units of K; the last may be partial (K % 8 == 0)
+    const int tail_chunks = (K & 63) >> 3;                   // 16-byte chunks of a row in a partial last unit (0: none)
     const int cnt = (KT - wave + 3) / 4;                     // units of this wave: wave, wave+4, ...
 
     const int rowsA = (M - row0) < BM ? (M - row0) : BM;
@@ -124,19 +126,25 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
                              : (uint32_t)((row - BM) * p.ldb + chunk * 8) * 2u;
     }
 
+    // In a partial last unit the chunks at k >= K belong to the next row of the matrix: the
+    // lanes that would fetch them ask for an offset past every descriptor instead and get zeros
+    // (the chunk a lane fetches depends on the parity of the instruction only: swz(8 * q + lr)).
+    const bool tail_ok[2] = {(lc ^ (lr >> 1)) < tail_chunks, (lc ^ (4 | (lr >> 1))) < tail_chunks};
     // unit i of this wave is unit wave + 4*i of the matrix; `rq_gs` follows the unit about to
     // be requested (requests past the last one fetch nothing), `rq_left` the live units left
     int rq_gs = wave;
     int rq_left = cnt;
     auto request = [&](int stage) __attribute__((always_inline)) {
         const bool live = rq_left > 0;
+        const bool tail = tail_chunks != 0 && rq_gs == KT - 1;
         --rq_left;
         const uint32_t kb = (uint32_t)rq_gs * 128u;
         rq_gs += 4;
         const uint32_t dst = ring_base + (uint32_t)(stage * STAGE);
 #pragma unroll
         for (int q = 0; q < L; ++q)
-            dma(live ? (q * 8 < BM ? rsrcA : rsrcB) : rsrcNone, voff[q] + kb, dst + (uint32_t)(q * 1024));
+            dma(live ? (q * 8 < BM ? rsrcA : rsrcB) : rsrcNone, (tail && !tail_ok[q & 1] ? 0x80000000u : voff[q]) + kb,
+                dst + (uint32_t)(q * 1024));
     };
 
     // fragment read: lane holds row l & 15 of a 16-row block, chunk 4*slice + (l >> 4)
@@ -266,7 +274,8 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
     int tm, tn;
     tile_of_block<4>(blockIdx.x, gridDim.x, tiles_m, tiles_n, tm, tn);
     const int row0 = tm * BM, col0 = tn * BN;
-    const int KT = K / 64;                                   // units of K
+    const int KT = (K + 63) / 64;                            // units of K; the last may be partial (K % 8 == 0)
+    const int tail_chunks = (K & 63) >> 3;                   // 16-byte chunks of a row in a partial last unit (0: none)
 
     const int rowsA = (M - row0) < BM ? (M - row0) : BM;
     const int rowsB = (N - col0) < BN ? (N - col0) : BN;
@@ -285,7 +294,9 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
     };
     auto swz = [](int row) __attribute__((always_inline)) { return (row >> 1) & 7; };
     // load instruction wave * LW + q of a unit fills stage rows 8 * that .. + 7 (A rows first,
-    // then B rows): this lane's byte offset inside A or B, k offset added per request
+    // then B rows): this lane's byte offset inside A or B, k offset added per request.
+    // In a partial last unit the chunks at k >= K belong to the next row of the matrix: the
+    // lanes that would fetch them ask for an offset past every descriptor instead and get zeros.
     const int lr = lane >> 3, lc = lane & 7;
     uint32_t voff[LW];
 #pragma unroll
@@ -295,16 +306,20 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
         voff[q] = row < BM ? (uint32_t)(row * p.lda + chunk * 8) * 2u
                            : (uint32_t)((row - BM) * p.ldb + chunk * 8) * 2u;
     }
+    // (the chunk a lane fetches depends on the parity of the instruction only: swz(8 * inst + lr))
+    const bool tail_ok[2] = {(lc ^ (lr >> 1)) < tail_chunks, (lc ^ (4 | (lr >> 1))) < tail_chunks};
     // `rq_unit` follows the unit about to be requested; requests past the last unit fetch nothing
     int rq_unit = 0;
     auto request = [&](int stage) __attribute__((always_inline)) {
         const bool live = rq_unit < KT;
+        const bool tail = tail_chunks != 0 && rq_unit == KT - 1;
         const uint32_t kb = (uint32_t)rq_unit * 128u;
         ++rq_unit;
         const uint32_t dst = lds_base + (uint32_t)(stage * STAGE + wave * LW * 1024);
 #pragma unroll
         for (int q = 0; q < LW; ++q)
-            dma(live ? ((wave * LW + q) * 8 < BM ? rsrcA : rsrcB) : rsrcNone, voff[q] + kb, dst + (uint32_t)(q * 1024));
+            dma(live ? ((wave * LW + q) * 8 < BM ? rsrcA : rsrcB) : rsrcNone,
+                (tail && !tail_ok[(wave * LW + q) & 1] ? 0x80000000u : voff[q]) + kb, dst + (uint32_t)(q * 1024));
     };
 
     // fragment read: lane holds row l & 15 of a 16-row block, chunk 4*slice + (l >> 4)

@@ -55,6 +55,11 @@ bool shape_is_streamable(int M, int N, int K, const void* A, const void* B, cons
     return N % 4 == 0 && K % 64 == 0 && aligned16(A) && aligned16(B) &&
            (((uintptr_t)C & 7u) == 0);
 }
+// The small-tile kernels fill a partial last K unit with zeros: rows of A and B that start on
+// 16-byte boundaries (K % 8 == 0) are all they need of K.
+bool shape_has_16_byte_rows(int N, int K, const void* A, const void* B, const void* C) {
+    return N % 4 == 0 && K % 8 == 0 && aligned16(A) && aligned16(B) && (((uintptr_t)C & 7u) == 0);
+}
 
 // Split-K geometry for a decode launch.  The decode kernel is bound by what one CU can pull
 // from HBM (~26 GB/s, whatever it keeps in flight), so it wants a workgroup on every CU: as
@@ -295,12 +300,12 @@ const std::vector<TunedEntry>& tuned_entries() {
     return table;
 }
 // config for (M, N, K) from the tuned file, or -1
-int tuned_config(int M, int N, int K, bool streamable) {
+int tuned_config(int M, int N, int K, bool streamable, bool rows16) {
     for (const TunedEntry& t : tuned_entries()) {
         if (t.M != M || t.N != N || t.K != K) continue;
         const mi::KernelEntry& e = mi::kKernels[t.config];
         if ((is_split_k_decode(e.kind) || e.kind == mi::KIND_STREAM) && (!streamable || M > e.BM)) continue;
-        if (e.kind == mi::KIND_WAVEK && !streamable) continue;
+        if (e.kind == mi::KIND_WAVEK && !rows16) continue;
         return t.config;
     }
     return -1;
@@ -319,7 +324,8 @@ Choice compute_choice(int requested, int M, int N, int K, bool streamable, bool 
     const int cus = compute_units();
     Choice c{M, N, K, flags, requested, cus, requested, 1, K};
     if (requested == MI_CONFIG_AUTO) {
-        c.config = tuned_config(M, N, K, streamable);
+        // (what the small-tile kernels need: select_kernel derives the same from its flags)
+        c.config = tuned_config(M, N, K, streamable, streamable || (splittable && ptr_aligned && K % 8 == 0));
         if (c.config < 0) c.config = mi::select_kernel(M, N, K, streamable, splittable, ptr_aligned, cus);
     }
     const mi::KernelEntry& e = mi::kKernels[c.config];
@@ -392,9 +398,9 @@ int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const vo
         return MI_OK;
     }
     if (e.kind == mi::KIND_WAVEK) {
-        if (!streamable)
+        if (!shape_has_16_byte_rows(N, K, A, B, C))
             return fail(MI_ERR_UNSUPPORTED,
-                        "config %s needs N %% 4 == 0, K %% 64 == 0 and 16-byte aligned operands", e.name);
+                        "config %s needs N %% 4 == 0, K %% 8 == 0 and 16-byte aligned operands", e.name);
         hipError_t err = e.launch[dtype][0](args, (hipStream_t)stream);
         if (err != hipSuccess)
             return fail(MI_ERR_HIP, "launch of %s failed: %s", e.name, hipGetErrorString(err));
@@ -489,7 +495,7 @@ int mi_gemm_config_supports(int config, int dtype, int M, int N, int K) {
     const mi::KernelEntry& e = mi::kKernels[config];
     if (is_split_k_decode(e.kind) || e.kind == mi::KIND_STREAM)
         return M <= e.BM && N % 4 == 0 && K % 64 == 0;
-    if (e.kind == mi::KIND_WAVEK) return N % 4 == 0 && K % 64 == 0;
+    if (e.kind == mi::KIND_WAVEK) return N % 4 == 0 && K % 8 == 0;
     if (e.kg > 1 && K % (128 * e.kg) != 0) return 0;
     return e.launch[dtype][1] != nullptr;
 }
@@ -504,7 +510,7 @@ int mi_gemm_config_grid(int config, int M, int N, int K) {
         return tiles_n * choose_splits(tiles_n, K, compute_units());
     }
     const int tiles = ((M + e.BM - 1) / e.BM) * ((N + e.BN - 1) / e.BN);
-    if (e.kind == mi::KIND_WAVEK) return K % 64 != 0 ? 0 : tiles;
+    if (e.kind == mi::KIND_WAVEK) return K % 8 != 0 ? 0 : tiles;
     if (e.kind == mi::KIND_MFMA16) {   // split-K pieces, assuming an aligned C and no trace buffer
         int kps = K;
         return tiles * choose_tile_splits(e, M, N, K, N % 4 == 0, true, compute_units(), &kps);
@@ -517,7 +523,7 @@ int mi_gemm_select_config(int dtype, int M, int N, int K) {
     if (!shape_in_range(M, N, K)) return -1;
     // pointer alignment is unknown here: assume the usual 256-byte aligned allocations
     const bool streamable = N % 4 == 0 && K % 64 == 0;
-    const int tuned = tuned_config(M, N, K, streamable);
+    const int tuned = tuned_config(M, N, K, streamable, N % 4 == 0 && K % 8 == 0);
     if (tuned >= 0) return tuned;
     return mi::select_kernel(M, N, K, streamable, N % 4 == 0, true, compute_units());
 }

@@ -218,8 +218,10 @@ def _s(BM, NS):
     return dict(KIND="stream", BM=BM, BN=32, NS=NS)
 
 
-def _k(BM, BN, NS, WK=None, OCC=1, SHARED=0):
+def _k(BM, BN, NS, WK=None, OCC=1, SHARED=0, WK_RAGGED=None):
     c = dict(KIND="wavek", BM=BM, BN=BN, NS=NS)
+    if WK_RAGGED is not None:
+        c["WK_RAGGED"] = WK_RAGGED     # a K unit's cost when K % 64 != 0, relative to an aligned pitch (default 1.45)
     if SHARED:
         c["SHARED"] = 1         # 2 x 2 waves over the tile and one ring, instead of K split over the waves
     if OCC != 1:
@@ -274,7 +276,7 @@ CONFIGS = [
     _k(64, 64, NS=1, OCC=2, WK=(1.93, 2.19, 0.1792, 0.0)),
     _k(64, 64, NS=2, WK=(0.88, 2.81, 0.1648, 0.0)),
     _k(96, 64, NS=2, WK=(1.35, 4.06, 0.2306, 0.0)),
-    _k(96, 96, NS=4, SHARED=1, WK=(1.23, 2.555, 0.3643, 0.0)),
+    _k(96, 96, NS=4, SHARED=1, WK=(1.23, 2.555, 0.3643, 0.0), WK_RAGGED=1.18),
     _k(64, 64, NS=4, SHARED=1, OCC=2, WK=(1.94, 1.270, 0.1847, 0.0)),
     _k(96, 64, NS=4, SHARED=1, OCC=2, WK=(2.58, 1.43, 0.2584, 0.0)),
     _k(64, 32, NS=4, SHARED=1, OCC=3, WK=(1.99, 0.958, 0.1252, 0.0)),

@@ -210,6 +210,14 @@ def test_wave_split_k_kernels(mi, orc, config):
     check_epilogue(mi, orc, 512, 512, 4096, "uniform", 0.37, 1.25, config=config)
     check_epilogue(mi, orc, 200, 132, 1024, "int", 2.0, -1.0, config=config, c_layout=mi.MI_C_COL_MAJOR, exact=True)
     # shapes the kernel cannot run are refused, not mis-computed
+    # a K of whole 16-byte chunks is enough: the partial last unit is filled with zeros (what
+    # lies at k >= K in memory is the next row), down to a single chunk and a single unit, the
+    # partial unit with each of the four waves
+    for M, N, K in [(bm, bn, 8), (97, 100, 72), (300, 260, 200), (1000, 1000, 1000), (1440, 1440, 1480),
+                    (33, 8, 456), (2 * bm - 1, 5 * bn - 4, 2168), (130, 132, 136), (130, 132, 248)]:
+        check(mi, orc, M, N, K, "int", config=config, exact=True)
+    check(mi, orc, 1000, 1000, 1000, "uniform", config=config)
+    check_epilogue(mi, orc, 300, 260, 1000, "int", -0.5, 2.75, config=config, exact=True)
     for M, N, K in [(256, 256, 100), (256, 254, 128)]:
         A, B = make_inputs(orc, M, N, K, "int")
         with pytest.raises(mi.MiGemmError) as ei:
@@ -393,6 +401,8 @@ def test_random_shapes_small_tile_and_decode_kinds(mi, orc):
         M = int(rng.choice([rng.integers(1, 130), rng.integers(1, 700)]))
         N = 4 * int(rng.integers(1, 180))
         K = 64 * int(rng.choice([1, 2, 3, rng.integers(4, 40)]))
+        if it % 4 == 1:
+            K = 8 * int(rng.integers(1, 300))     # whole 16-byte chunks only: the small-tile kernels still run
         offA, offB, offC = 16 * int(rng.integers(0, 4)), 16 * int(rng.integers(0, 4)), 8 * int(rng.integers(0, 8))
         able = [i for i in special if mi._lib.load().mi_gemm_config_supports(i, 0, M, N, K)]
         config = -1 if it % 3 == 0 or not able else able[int(rng.integers(0, len(able)))]

@@ -201,8 +201,9 @@ def test_config_table(mi):
     assert picked(4095, 6143, 3073) == (256, 192)
     assert picked(512, 512, 512) == (32, 32)
     assert kc.CONFIGS[mi.select_config(512, 512, 512)]['KIND'] == 'wavek'
-    assert picked(512, 512, 520) == (128, 128)
-    assert kc.CONFIGS[mi.select_config(512, 512, 520)]['KIND'] == 'mfma16'
+    assert picked(512, 512, 522) == (128, 128)
+    assert kc.CONFIGS[mi.select_config(512, 512, 522)]['KIND'] == 'mfma16'
+    assert kc.CONFIGS[mi.select_config(512, 512, 520)]['KIND'] == 'wavek'      # rows that start on 16-byte boundaries are enough for the small-tile kernels
     assert all("EFF" in kc.CONFIGS[mi.select_config(M, N, 4100)] for M in (257, 1000, 5000) for N in (100, 3000))
     # few tiles and a long K: split-K pieces of a tiled kernel fill the CUs
     c = mi.select_config(256, 8192, 8192)
@@ -211,7 +212,7 @@ def test_config_table(mi):
     c = mi.find_config("m128x128_w2x2_g4_b1_o2")                    # (the automatic choice is the small-tile kernel)
     assert mi.config_grid(c, 512, 512, 4096) == 16 * 8              # 128x128 tiles x 8 pieces of 512
     assert mi.config_grid(mi.select_config(8192, 8192, 8192), 8192, 8192, 8192) == 1024   # no split-K when the tiles fill the chip
-    assert mi.config_grid(mi.select_config(512, 512, 520), 512, 512, 520) == 16           # nor for a short K
+    assert mi.config_grid(mi.select_config(512, 512, 522), 512, 512, 522) == 16           # nor for a short K
     assert mi.config_grid(mi.select_config(512, 512, 512), 512, 512, 512) == 256          # 32x32 tiles, one per CU
     c = mi.select_config(512, 510, 4096)
     assert mi.config_grid(c, 512, 510, 4096) == -(-512 // kc.CONFIGS[c]["BM"]) * -(-510 // kc.CONFIGS[c]["BN"])   # N % 4 != 0: no split-K
