@@ -43,9 +43,12 @@
 // single stage and one workgroup per CU only, were far behind the tiled kernels (2048^3:
 // 26.5 us against 19.6): alone and with one stage, loading and multiplying take turns.
 // Rows of A past M and rows of B past N are never fetched (the buffer descriptors end at the
-// last valid row of the tile).  Preconditions, checked by the launcher's caller: K % 8 == 0 and
-// 16-byte aligned A and B (rows that start on 16-byte boundaries; a partial last unit of K is
-// filled up with zeros), N % 4 == 0, 8-byte aligned C.
+// last valid row of the tile).  Preconditions, checked by the launcher's caller: K even and
+// 4-byte aligned A and B (rows of whole 32-bit words, which is what the descriptors' range check
+// counts in; a partial last unit of K is filled up with zeros).  Any N and any C: where the
+// groups of four elements do not all start on 8-byte boundaries inside N, C is stored element
+// by element.  Rows that start on 128-byte boundaries (K % 64 == 0, aligned bases) are what the
+// kernel is fastest on: with any other pitch every 128-byte piece of a row straddles two lines.
 // The reference has no counterpart: its kernels use one tile size (matmul_utils.cuh:362).
 #pragma once
 
@@ -57,6 +60,18 @@
 #include "splitk_common.hpp"        // DecodeArgs
 
 namespace mi {
+
+// K tail inside a 16-byte chunk (K % 8 != 0, K even).  The chunk of a row that holds k = K - 1
+// also holds the first elements of the next row of the matrix; the lane that fetched it keeps
+// its K % 8 leading elements and zeroes the rest, in LDS, once its loads of that unit have
+// landed and before anyone reads the stage.  `ptr`: the 16 bytes this lane's load wrote.
+__device__ __forceinline__ void zero_chunk_tail(unsigned char* ptr, int keep_elems) {
+    u32x4_t v = *(const u32x4_t*)ptr;
+    const int keep_words = keep_elems >> 1;                  // K is even: whole 32-bit words
+#pragma unroll
+    for (int w = 0; w < 4; ++w) v[w] = w < keep_words ? v[w] : 0u;
+    *(u32x4_t*)ptr = v;
+}
 
 template <int BM_, int BN_, int NS_, int DT_>
 struct WaveKConfig {
@@ -93,8 +108,9 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
     int tm, tn;
     tile_of_block<4>(blockIdx.x, gridDim.x, tiles_m, tiles_n, tm, tn);
     const int row0 = tm * BM, col0 = tn * BN;
-    const int KT = (K + 63) / 64;                            // units of K; the last may be partial (K % 8 == 0)
-    const int tail_chunks = (K & 63) >> 3;                   // 16-byte chunks of a row in a partial last unit (0: none)
+    const int KT = (K + 63) / 64;                            // units of K; the last may be partial (K even)
+    const int tail_chunks = ((K & 63) + 7) >> 3;             // 16-byte chunks of a row in a partial last unit (0: none)
+    const int tail_elems = K & 7;                            // elements of k < K in the last of them (0: all eight)
     const int cnt = (KT - wave + 3) / 4;                     // units of this wave: wave, wave+4, ...
 
     const int rowsA = (M - row0) < BM ? (M - row0) : BM;
@@ -167,6 +183,14 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
     for (int u = 0; u < cnt; ++u) {
         // unit u of this wave has landed
         asm volatile("s_waitcnt vmcnt(%0)" :: "n"((NS - 1) * L) : "memory");
+        if (tail_elems != 0 && wave + 4 * u == KT - 1) {
+            // the matrix's last unit ends inside a chunk: each lane looks after what it fetched
+#pragma unroll
+            for (int q = 0; q < L; ++q)
+                if ((lc ^ (((q & 1) << 2) | (lr >> 1))) == tail_chunks - 1)
+                    zero_chunk_tail(lds + wave * REGION + s * STAGE + q * 1024 + lane * 16, tail_elems);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        }
         const unsigned char* st = ring + s * STAGE;
         u32x4_t fa[2][MI], fb[2][NI];
 #pragma unroll
@@ -201,6 +225,7 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
             *(f32x4_t*)(part + (i * 16 + l16) * PITCH + j * 16 + 4 * q4) = acc[i][j];
     __syncthreads();
     const bool scaled = p.alpha != 1.0f || p.beta != 0.0f;
+    const bool c_vec_ok = (N & 3) == 0 && (p.ldc & 3) == 0 && ((uintptr_t)p.C & 7u) == 0;
 #pragma unroll
     for (int it = 0; it < Cfg::QUADS; ++it) {
         const int q = it * 256 + tid;
@@ -215,11 +240,18 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) sum[e] = mul_add_unfused(sum[e], p.alpha, p.beta);
         }
-        if (row0 + m < M && col0 + n < N) {                  // N % 4 == 0 is a launch precondition
+        if (row0 + m < M && col0 + n < N) {
             u32x2_t w2;
             w2[0] = cvt_store2<DT>(sum[0], sum[1]);
             w2[1] = cvt_store2<DT>(sum[2], sum[3]);
-            *(u32x2_t*)((unsigned char*)p.C + ((size_t)(row0 + m) * p.ldc + col0 + n) * 2) = w2;
+            unsigned char* dst = (unsigned char*)p.C + ((size_t)(row0 + m) * p.ldc + col0 + n) * 2;
+            if (c_vec_ok) {                                  // every group of four starts on an 8-byte boundary inside N
+                *(u32x2_t*)dst = w2;
+            } else {                                         // any N, any 2-byte aligned C: element by element
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (col0 + n + e < N) ((uint16_t*)dst)[e] = (uint16_t)(w2[e >> 1] >> ((e & 1) * 16));
+            }
         }
     }
 }
@@ -274,8 +306,9 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
     int tm, tn;
     tile_of_block<4>(blockIdx.x, gridDim.x, tiles_m, tiles_n, tm, tn);
     const int row0 = tm * BM, col0 = tn * BN;
-    const int KT = (K + 63) / 64;                            // units of K; the last may be partial (K % 8 == 0)
-    const int tail_chunks = (K & 63) >> 3;                   // 16-byte chunks of a row in a partial last unit (0: none)
+    const int KT = (K + 63) / 64;                            // units of K; the last may be partial (K even)
+    const int tail_chunks = ((K & 63) + 7) >> 3;             // 16-byte chunks of a row in a partial last unit (0: none)
+    const int tail_elems = K & 7;                            // elements of k < K in the last of them (0: all eight)
 
     const int rowsA = (M - row0) < BM ? (M - row0) : BM;
     const int rowsB = (N - col0) < BN ? (N - col0) : BN;
@@ -355,12 +388,27 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
         }
     };
     int s = 0;                                               // stage of the unit being multiplied
+    int landed = 0;                                          // the unit whose landing the next barrier publishes
+    // the matrix's last unit ends inside a chunk: each lane looks after what it fetched, after its
+    // loads of that unit have landed and before the barrier that lets everyone read the stage
+    auto fix_tail = [&](int stage) __attribute__((always_inline)) {
+        if (tail_elems != 0 && landed == KT - 1) {
+#pragma unroll
+            for (int q = 0; q < LW; ++q)
+                if ((lc ^ ((((wave * LW + q) & 1) << 2) | (lr >> 1))) == tail_chunks - 1)
+                    zero_chunk_tail(lds + stage * STAGE + (wave * LW + q) * 1024 + lane * 16, tail_elems);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        }
+        ++landed;
+    };
     // one step: unit u (fragments in set CUR) is multiplied while unit u + 1 is read into the other set
     auto step = [&](auto cur_c) __attribute__((always_inline)) {
         constexpr int CUR = decltype(cur_c)::value;
         // this wave's loads of unit u + 1 have landed; after the barrier everyone's have, and
         // everyone has multiplied unit u - 1, whose stage takes the request NS - 1 units ahead
-        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"((NS - 3) * LW) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0)" :: "n"((NS - 3) * LW) : "memory");
+        fix_tail(s + 1 == NS ? 0 : s + 1);
+        asm volatile("s_barrier" ::: "memory");
         request(s == 0 ? NS - 1 : s - 1);
         read_unit(s + 1 == NS ? 0 : s + 1, fa[CUR ^ 1], fb[CUR ^ 1]);   // (past the last unit: zeros or stale rows, never multiplied)
         __builtin_amdgcn_sched_barrier(0);
@@ -374,7 +422,9 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
         __builtin_amdgcn_sched_barrier(0);
         s = s + 1 == NS ? 0 : s + 1;
     };
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"((NS - 2) * LW) : "memory");     // unit 0 has landed
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"((NS - 2) * LW) : "memory");     // unit 0 has landed
+    fix_tail(0);
+    asm volatile("s_barrier" ::: "memory");
     read_unit(0, fa[0], fb[0]);
     int u = 0;
     for (; u + 2 <= KT; u += 2) {
@@ -396,6 +446,7 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
             *(f32x4_t*)(part + (wm * TM + i * 16 + l16) * PITCH + wn * TN + j * 16 + 4 * q4) = acc[i][j];
     __syncthreads();
     const bool scaled = p.alpha != 1.0f || p.beta != 0.0f;
+    const bool c_vec_ok = (N & 3) == 0 && (p.ldc & 3) == 0 && ((uintptr_t)p.C & 7u) == 0;
 #pragma unroll
     for (int it = 0; it < Cfg::QUADS; ++it) {
         const int q = it * 256 + tid;
@@ -405,11 +456,18 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
 #pragma unroll
             for (int e = 0; e < 4; ++e) sum[e] = mul_add_unfused(sum[e], p.alpha, p.beta);
         }
-        if (row0 + m < M && col0 + n < N) {                  // N % 4 == 0 is a launch precondition
+        if (row0 + m < M && col0 + n < N) {
             u32x2_t w2;
             w2[0] = cvt_store2<DT>(sum[0], sum[1]);
             w2[1] = cvt_store2<DT>(sum[2], sum[3]);
-            *(u32x2_t*)((unsigned char*)p.C + ((size_t)(row0 + m) * p.ldc + col0 + n) * 2) = w2;
+            unsigned char* dst = (unsigned char*)p.C + ((size_t)(row0 + m) * p.ldc + col0 + n) * 2;
+            if (c_vec_ok) {                                  // every group of four starts on an 8-byte boundary inside N
+                *(u32x2_t*)dst = w2;
+            } else {                                         // any N, any 2-byte aligned C: element by element
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (col0 + n + e < N) ((uint16_t*)dst)[e] = (uint16_t)(w2[e >> 1] >> ((e & 1) * 16));
+            }
         }
     }
 }

@@ -55,10 +55,11 @@ bool shape_is_streamable(int M, int N, int K, const void* A, const void* B, cons
     return N % 4 == 0 && K % 64 == 0 && aligned16(A) && aligned16(B) &&
            (((uintptr_t)C & 7u) == 0);
 }
-// The small-tile kernels fill a partial last K unit with zeros: rows of A and B that start on
-// 16-byte boundaries (K % 8 == 0) are all they need of K.
-bool shape_has_16_byte_rows(int N, int K, const void* A, const void* B, const void* C) {
-    return N % 4 == 0 && K % 8 == 0 && aligned16(A) && aligned16(B) && (((uintptr_t)C & 7u) == 0);
+// The small-tile kernels fill a partial last K unit with zeros and store a C of any N and
+// alignment: rows of A and B made of whole 32-bit words (K even, 4-byte aligned bases) are all
+// they need.
+bool shape_has_word_rows(int K, const void* A, const void* B) {
+    return K % 2 == 0 && (((uintptr_t)A | (uintptr_t)B) & 3u) == 0;
 }
 
 // Split-K geometry for a decode launch.  The decode kernel is bound by what one CU can pull
@@ -300,12 +301,12 @@ const std::vector<TunedEntry>& tuned_entries() {
     return table;
 }
 // config for (M, N, K) from the tuned file, or -1
-int tuned_config(int M, int N, int K, bool streamable, bool rows16) {
+int tuned_config(int M, int N, int K, bool streamable, bool small_ok) {
     for (const TunedEntry& t : tuned_entries()) {
         if (t.M != M || t.N != N || t.K != K) continue;
         const mi::KernelEntry& e = mi::kKernels[t.config];
         if ((is_split_k_decode(e.kind) || e.kind == mi::KIND_STREAM) && (!streamable || M > e.BM)) continue;
-        if (e.kind == mi::KIND_WAVEK && !rows16) continue;
+        if (e.kind == mi::KIND_WAVEK && !small_ok) continue;
         return t.config;
     }
     return -1;
@@ -319,14 +320,14 @@ struct Choice {
     int M, N, K, flags, requested, cus;   // key; requested = the caller's config (MI_CONFIG_AUTO or an index)
     int config, splits, k_per_split;
 };
-Choice compute_choice(int requested, int M, int N, int K, bool streamable, bool splittable, bool ptr_aligned) {
-    const int flags = (streamable ? 1 : 0) | (splittable ? 2 : 0) | (ptr_aligned ? 4 : 0);
+Choice compute_choice(int requested, int M, int N, int K, bool streamable, bool splittable, bool ptr_aligned,
+                      bool small_ok) {
+    const int flags = (streamable ? 1 : 0) | (splittable ? 2 : 0) | (ptr_aligned ? 4 : 0) | (small_ok ? 8 : 0);
     const int cus = compute_units();
     Choice c{M, N, K, flags, requested, cus, requested, 1, K};
     if (requested == MI_CONFIG_AUTO) {
-        // (what the small-tile kernels need: select_kernel derives the same from its flags)
-        c.config = tuned_config(M, N, K, streamable, streamable || (splittable && ptr_aligned && K % 8 == 0));
-        if (c.config < 0) c.config = mi::select_kernel(M, N, K, streamable, splittable, ptr_aligned, cus);
+        c.config = tuned_config(M, N, K, streamable, small_ok);
+        if (c.config < 0) c.config = mi::select_kernel(M, N, K, streamable, splittable, ptr_aligned, small_ok, cus);
     }
     const mi::KernelEntry& e = mi::kKernels[c.config];
     if (e.kind == mi::KIND_MFMA16) {
@@ -338,16 +339,16 @@ Choice compute_choice(int requested, int M, int N, int K, bool streamable, bool 
     }
     return c;
 }
-Choice choose(int requested, int M, int N, int K, bool streamable, bool splittable, bool ptr_aligned) {
+Choice choose(int requested, int M, int N, int K, bool streamable, bool splittable, bool ptr_aligned, bool small_ok) {
     static thread_local Choice memo[4] = {};
     static thread_local int next = 0;
-    const int flags = (streamable ? 1 : 0) | (splittable ? 2 : 0) | (ptr_aligned ? 4 : 0);
+    const int flags = (streamable ? 1 : 0) | (splittable ? 2 : 0) | (ptr_aligned ? 4 : 0) | (small_ok ? 8 : 0);
     const int cus = compute_units();
     for (const Choice& c : memo)
         if (c.M == M && c.N == N && c.K == K && c.flags == flags && c.requested == requested && c.cus == cus &&
             c.splits > 0)
             return c;
-    const Choice c = compute_choice(requested, M, N, K, streamable, splittable, ptr_aligned);
+    const Choice c = compute_choice(requested, M, N, K, streamable, splittable, ptr_aligned, small_ok);
     memo[next] = c;
     next = (next + 1) & 3;
     return c;
@@ -363,7 +364,8 @@ int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const vo
     // ones); an explicitly requested decode or small-tile kernel runs and leaves it untouched
     const Choice choice = choose(config, M, N, K, streamable && !(config == MI_CONFIG_AUTO && DB),
                                  shape_is_splittable(N, C, DB),
-                                 aligned16(A) && aligned16(B) && aligned16(C));
+                                 aligned16(A) && aligned16(B) && aligned16(C),
+                                 shape_has_word_rows(K, A, B) && !(config == MI_CONFIG_AUTO && DB));
     config = choice.config;
     const mi::KernelEntry& e = mi::kKernels[config];
 
@@ -398,9 +400,8 @@ int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const vo
         return MI_OK;
     }
     if (e.kind == mi::KIND_WAVEK) {
-        if (!shape_has_16_byte_rows(N, K, A, B, C))
-            return fail(MI_ERR_UNSUPPORTED,
-                        "config %s needs N %% 4 == 0, K %% 8 == 0 and 16-byte aligned operands", e.name);
+        if (!shape_has_word_rows(K, A, B))
+            return fail(MI_ERR_UNSUPPORTED, "config %s needs an even K and 4-byte aligned A and B", e.name);
         hipError_t err = e.launch[dtype][0](args, (hipStream_t)stream);
         if (err != hipSuccess)
             return fail(MI_ERR_HIP, "launch of %s failed: %s", e.name, hipGetErrorString(err));
@@ -495,7 +496,7 @@ int mi_gemm_config_supports(int config, int dtype, int M, int N, int K) {
     const mi::KernelEntry& e = mi::kKernels[config];
     if (is_split_k_decode(e.kind) || e.kind == mi::KIND_STREAM)
         return M <= e.BM && N % 4 == 0 && K % 64 == 0;
-    if (e.kind == mi::KIND_WAVEK) return N % 4 == 0 && K % 8 == 0;
+    if (e.kind == mi::KIND_WAVEK) return K % 2 == 0;
     if (e.kg > 1 && K % (128 * e.kg) != 0) return 0;
     return e.launch[dtype][1] != nullptr;
 }
@@ -510,7 +511,7 @@ int mi_gemm_config_grid(int config, int M, int N, int K) {
         return tiles_n * choose_splits(tiles_n, K, compute_units());
     }
     const int tiles = ((M + e.BM - 1) / e.BM) * ((N + e.BN - 1) / e.BN);
-    if (e.kind == mi::KIND_WAVEK) return K % 8 != 0 ? 0 : tiles;
+    if (e.kind == mi::KIND_WAVEK) return K % 2 != 0 ? 0 : tiles;
     if (e.kind == mi::KIND_MFMA16) {   // split-K pieces, assuming an aligned C and no trace buffer
         int kps = K;
         return tiles * choose_tile_splits(e, M, N, K, N % 4 == 0, true, compute_units(), &kps);
@@ -523,9 +524,9 @@ int mi_gemm_select_config(int dtype, int M, int N, int K) {
     if (!shape_in_range(M, N, K)) return -1;
     // pointer alignment is unknown here: assume the usual 256-byte aligned allocations
     const bool streamable = N % 4 == 0 && K % 64 == 0;
-    const int tuned = tuned_config(M, N, K, streamable, N % 4 == 0 && K % 8 == 0);
+    const int tuned = tuned_config(M, N, K, streamable, K % 2 == 0);
     if (tuned >= 0) return tuned;
-    return mi::select_kernel(M, N, K, streamable, N % 4 == 0, true, compute_units());
+    return mi::select_kernel(M, N, K, streamable, N % 4 == 0, true, K % 2 == 0, compute_units());
 }
 
 int mi_gemm_tuned_entries(void) { return (int)tuned_entries().size(); }
@@ -578,9 +579,13 @@ size_t mi_gemm_workspace_bytes(int config, int dtype, int M, int N, int K, int c
     const bool can_stream = N % 4 == 0 && K % 64 == 0;
     for (int aligned = 0; aligned < 2; ++aligned)
         for (int streamable = 0; streamable < (can_stream && aligned ? 2 : 1); ++streamable) {
-            const Choice c = compute_choice(config, M, N, K, streamable != 0, N % 4 == 0, aligned != 0);
+            // (a launch that cannot use the small-tile kernels -- operands not 4-byte aligned -- may split where
+            // one that can does not: both cases)
+            for (int small = 0; small < (K % 2 == 0 ? 2 : 1); ++small) {
+            const Choice c = compute_choice(config, M, N, K, streamable != 0, N % 4 == 0, aligned != 0, small != 0);
             const size_t b = c.splits > 1 ? (size_t)c.splits * M * N * sizeof(float) : 0;
             if (b > need) need = b;
+            }
         }
     return need;
 }

@@ -210,15 +210,23 @@ def test_wave_split_k_kernels(mi, orc, config):
     check_epilogue(mi, orc, 512, 512, 4096, "uniform", 0.37, 1.25, config=config)
     check_epilogue(mi, orc, 200, 132, 1024, "int", 2.0, -1.0, config=config, c_layout=mi.MI_C_COL_MAJOR, exact=True)
     # shapes the kernel cannot run are refused, not mis-computed
-    # a K of whole 16-byte chunks is enough: the partial last unit is filled with zeros (what
-    # lies at k >= K in memory is the next row), down to a single chunk and a single unit, the
-    # partial unit with each of the four waves
+    # any even K: the partial last unit is filled with zeros (what lies at k >= K in memory is
+    # the next row) -- whole 16-byte chunks by fetching nothing, the chunk that K ends in by
+    # zeroing its tail in LDS -- down to a single chunk and a single unit, the partial unit with
+    # each of the four waves; any N (C stored element by element where rows of C do not start on
+    # 8-byte boundaries)
     for M, N, K in [(bm, bn, 8), (97, 100, 72), (300, 260, 200), (1000, 1000, 1000), (1440, 1440, 1480),
-                    (33, 8, 456), (2 * bm - 1, 5 * bn - 4, 2168), (130, 132, 136), (130, 132, 248)]:
+                    (33, 8, 456), (2 * bm - 1, 5 * bn - 4, 2168), (130, 132, 136), (130, 132, 248),
+                    (bm, bn, 2), (bm + 3, bn + 1, 6), (97, 101, 66), (300, 259, 100), (500, 500, 500),
+                    (1500, 1500, 1500), (255, 1001, 1030), (130, 130, 190), (7, 3, 254), (640, 77, 4100)]:
         check(mi, orc, M, N, K, "int", config=config, exact=True)
     check(mi, orc, 1000, 1000, 1000, "uniform", config=config)
+    check(mi, orc, 1500, 1002, 1500, "uniform", config=config)
+    check(mi, orc, 300, 201, 500, "normal", config=config, dtype=orc.FP16)
     check_epilogue(mi, orc, 300, 260, 1000, "int", -0.5, 2.75, config=config, exact=True)
-    for M, N, K in [(256, 256, 100), (256, 254, 128)]:
+    check_epilogue(mi, orc, 300, 261, 1002, "int", -0.5, 2.75, config=config, exact=True)
+    check_epilogue(mi, orc, 200, 131, 1026, "int", 2.0, -1.0, config=config, c_layout=mi.MI_C_COL_MAJOR, exact=True)
+    for M, N, K in [(256, 256, 101), (256, 254, 1)]:
         A, B = make_inputs(orc, M, N, K, "int")
         with pytest.raises(mi.MiGemmError) as ei:
             Dev(mi, A, B, M, N).run(K, config=config)
@@ -396,18 +404,25 @@ def test_random_shapes_small_tile_and_decode_kinds(mi, orc):
     from h100_gemm_amd import kernel_configs as kc
     rng = np.random.default_rng(20241125)
     special = [i for i, c in enumerate(kc.CONFIGS) if c["KIND"] in ("wavek", "stream", "decode")]
+    small = [i for i, c in enumerate(kc.CONFIGS) if c["KIND"] == "wavek"]
     # MI_GEMM_RANDOM_CASES=<n> turns this into a longer sweep (36 cases by default)
     for it in range(int(os.environ.get("MI_GEMM_RANDOM_CASES", "36"))):
         M = int(rng.choice([rng.integers(1, 130), rng.integers(1, 700)]))
         N = 4 * int(rng.integers(1, 180))
         K = 64 * int(rng.choice([1, 2, 3, rng.integers(4, 40)]))
-        if it % 4 == 1:
-            K = 8 * int(rng.integers(1, 300))     # whole 16-byte chunks only: the small-tile kernels still run
         offA, offB, offC = 16 * int(rng.integers(0, 4)), 16 * int(rng.integers(0, 4)), 8 * int(rng.integers(0, 8))
-        able = [i for i in special if mi._lib.load().mi_gemm_config_supports(i, 0, M, N, K)]
+        pool = special
+        if it % 2 == 1:
+            # what only the small-tile kernels take: any even K, any N, operands on 4-byte and C on
+            # 2-byte boundaries
+            K = 2 * int(rng.choice([rng.integers(1, 40), rng.integers(40, 1300)]))
+            N = int(rng.integers(1, 720))
+            offA, offB, offC = 4 * int(rng.integers(0, 16)), 4 * int(rng.integers(0, 16)), 2 * int(rng.integers(0, 32))
+            pool = small
+        able = [i for i in pool if mi._lib.load().mi_gemm_config_supports(i, 0, M, N, K)]
         config = -1 if it % 3 == 0 or not able else able[int(rng.integers(0, len(able)))]
         if it % 7 == 3:
-            config, offA = -1, offA + 2          # not 16-byte aligned: none of these kernels may be chosen
+            config, offA = -1, offA + 2          # not 4-byte aligned: none of these kernels may be chosen
         print(f"case {it}: M={M} N={N} K={K} offsets {offA},{offB},{offC} config={config}", flush=True)
         C, ref, guard = _run_offset(mi, orc, config, M, N, K, offA, offB, offC)
         assert (C == ref).all(), f"{int((C != ref).sum())} elements differ"

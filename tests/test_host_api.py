@@ -146,12 +146,12 @@ def test_config_table(mi):
             assert mi.config_grid(i, 16, 8192, 8192) >= 64
             assert mi.config_grid(i, c["BM"] + 1, 8192, 8192) == 0
         elif c["KIND"] == "wavek":
-            # any M; whole 64-deep K units, N a multiple of 4; no ragged twin
+            # any M and N; rows of whole 32-bit words (an even K); no ragged twin
             assert mi.config_grid(i, 1000, 780, 64) == -(-1000 // c["BM"]) * -(-780 // c["BN"])
             assert L.mi_gemm_config_supports(i, 0, 1000, 780, 4096) == 1
-            assert L.mi_gemm_config_supports(i, 0, 1000, 780, 4100) == 0
-            assert L.mi_gemm_config_supports(i, 0, 1000, 778, 4096) == 0
-            assert mi.config_grid(i, 1000, 780, 4100) == 0
+            assert L.mi_gemm_config_supports(i, 0, 1000, 777, 4098) == 1
+            assert L.mi_gemm_config_supports(i, 0, 1000, 780, 4097) == 0
+            assert mi.config_grid(i, 1000, 780, 4097) == 0
         elif c.get("KG", 1) > 1:
             # K split over groups of waves inside the workgroup: any M, N; K in equal halves of whole double steps
             assert L.mi_gemm_config_supports(i, 0, 4095, 6143, 3072) == 1
@@ -180,8 +180,9 @@ def test_config_table(mi):
     # few tiles and a long K: small tiles with K split over the waves, when the kernel can run the shape
     assert kc.CONFIGS[mi.select_config(512, 512, 4096)]["KIND"] == "wavek"
     assert kc.CONFIGS[mi.select_config(1024, 1024, 4096)]["KIND"] == "wavek"
-    assert kc.CONFIGS[mi.select_config(512, 512, 4100)]["KIND"] == "mfma16"
-    assert kc.CONFIGS[mi.select_config(512, 510, 4096)]["KIND"] == "mfma16"
+    assert kc.CONFIGS[mi.select_config(512, 512, 4100)]["KIND"] == "wavek"     # an even K and any N will do
+    assert kc.CONFIGS[mi.select_config(512, 510, 4096)]["KIND"] == "wavek"
+    assert kc.CONFIGS[mi.select_config(512, 512, 4101)]["KIND"] == "mfma16"    # an odd K: the predicated tiled kernels
     # a mid-sized output with a K of moderate length: small tiles on a shared ring (K is not split
     # over the waves), also with a short K and many tiles, where the K-splitting ones are shut out
     assert not kc.CONFIGS[mi.select_config(512, 512, 4096)].get("SHARED")
@@ -192,7 +193,7 @@ def test_config_table(mi):
     # wave quantisation: 256 CUs; 8192^2 fills four rounds of 256x256 tiles, 4095x6143 fills
     # two rounds of 256x192 tiles exactly (256x256 would leave half of the second round
     # idle), and 512^2 is a single partial round whatever the tiled kernel: the small-tile
-    # kernel gives every CU a 32x32 tile (one with a ragged K cannot run it: 128x128 tiles)
+    # kernel gives every CU a 32x32 tile (one with an odd K cannot run it: 128x128 tiles)
     def picked(M, N, K):
         c = kc.CONFIGS[mi.select_config(M, N, K)]
         return c["BM"], c["BN"]
@@ -201,10 +202,10 @@ def test_config_table(mi):
     assert picked(4095, 6143, 3073) == (256, 192)
     assert picked(512, 512, 512) == (32, 32)
     assert kc.CONFIGS[mi.select_config(512, 512, 512)]['KIND'] == 'wavek'
-    assert picked(512, 512, 522) == (128, 128)
-    assert kc.CONFIGS[mi.select_config(512, 512, 522)]['KIND'] == 'mfma16'
-    assert kc.CONFIGS[mi.select_config(512, 512, 520)]['KIND'] == 'wavek'      # rows that start on 16-byte boundaries are enough for the small-tile kernels
-    assert all("EFF" in kc.CONFIGS[mi.select_config(M, N, 4100)] for M in (257, 1000, 5000) for N in (100, 3000))
+    assert picked(512, 512, 521) == (128, 128)
+    assert kc.CONFIGS[mi.select_config(512, 512, 521)]['KIND'] == 'mfma16'
+    assert kc.CONFIGS[mi.select_config(512, 512, 522)]['KIND'] == 'wavek'      # rows of whole 32-bit words are enough for the small-tile kernels
+    assert all("EFF" in kc.CONFIGS[mi.select_config(M, N, 4101)] for M in (257, 1000, 5000) for N in (100, 3000))
     # few tiles and a long K: split-K pieces of a tiled kernel fill the CUs
     c = mi.select_config(256, 8192, 8192)
     assert kc.CONFIGS[c]["KIND"] == "mfma16" and (kc.CONFIGS[c]["BM"], kc.CONFIGS[c]["BN"]) == (256, 128)
@@ -212,10 +213,10 @@ def test_config_table(mi):
     c = mi.find_config("m128x128_w2x2_g4_b1_o2")                    # (the automatic choice is the small-tile kernel)
     assert mi.config_grid(c, 512, 512, 4096) == 16 * 8              # 128x128 tiles x 8 pieces of 512
     assert mi.config_grid(mi.select_config(8192, 8192, 8192), 8192, 8192, 8192) == 1024   # no split-K when the tiles fill the chip
-    assert mi.config_grid(mi.select_config(512, 512, 522), 512, 512, 522) == 16           # nor for a short K
+    assert mi.config_grid(mi.select_config(512, 512, 521), 512, 512, 521) == 16           # nor for a short K
     assert mi.config_grid(mi.select_config(512, 512, 512), 512, 512, 512) == 256          # 32x32 tiles, one per CU
-    c = mi.select_config(512, 510, 4096)
-    assert mi.config_grid(c, 512, 510, 4096) == -(-512 // kc.CONFIGS[c]["BM"]) * -(-510 // kc.CONFIGS[c]["BN"])   # N % 4 != 0: no split-K
+    c = mi.select_config(512, 510, 4097)
+    assert mi.config_grid(c, 512, 510, 4097) == -(-512 // kc.CONFIGS[c]["BM"]) * -(-510 // kc.CONFIGS[c]["BN"])   # N % 4 != 0: no split-K
     assert "EFF" in kc.CONFIGS[mi.select_config(200, 8190, 8192)]        # N % 4 != 0: tiled
     assert not kc.is_valid_config(dict(KIND="tile", BM=256, BN=256, WM=2, WN=2, SWZ=1, GROUP=8, OCC=2, DTL=0, EPI=0))
     assert not kc.is_valid_config(dict(KIND="tile", BM=96, BN=256, WM=2, WN=2, SWZ=1, GROUP=8, OCC=1, DTL=0, EPI=0))
