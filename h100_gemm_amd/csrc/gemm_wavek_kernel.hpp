@@ -145,7 +145,7 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
     // In a partial last unit the chunks at k >= K belong to the next row of the matrix: the
     // lanes that would fetch them ask for an offset past every descriptor instead and get zeros
     // (the chunk a lane fetches depends on the parity of the instruction only: swz(8 * q + lr)).
-    const bool tail_ok[2] = {(lc ^ (lr >> 1)) < tail_chunks, (lc ^ (4 | (lr >> 1))) < tail_chunks};
+    const bool tail_ok_even = (lc ^ (lr >> 1)) < tail_chunks, tail_ok_odd = (lc ^ (4 | (lr >> 1))) < tail_chunks;
     // unit i of this wave is unit wave + 4*i of the matrix; `rq_gs` follows the unit about to
     // be requested (requests past the last one fetch nothing), `rq_left` the live units left
     int rq_gs = wave;
@@ -157,10 +157,16 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
         const uint32_t kb = (uint32_t)rq_gs * 128u;
         rq_gs += 4;
         const uint32_t dst = ring_base + (uint32_t)(stage * STAGE);
+        if (!tail) {
 #pragma unroll
-        for (int q = 0; q < L; ++q)
-            dma(live ? (q * 8 < BM ? rsrcA : rsrcB) : rsrcNone, (tail && !tail_ok[q & 1] ? 0x80000000u : voff[q]) + kb,
-                dst + (uint32_t)(q * 1024));
+            for (int q = 0; q < L; ++q)
+                dma(live ? (q * 8 < BM ? rsrcA : rsrcB) : rsrcNone, voff[q] + kb, dst + (uint32_t)(q * 1024));
+        } else {                                             // (a path of its own: nothing of it in the other units' way)
+#pragma unroll
+            for (int q = 0; q < L; ++q)
+                dma(q * 8 < BM ? rsrcA : rsrcB, ((q & 1) ? tail_ok_odd : tail_ok_even) ? voff[q] + kb : 0x80000000u,
+                    dst + (uint32_t)(q * 1024));
+        }
     };
 
     // fragment read: lane holds row l & 15 of a 16-row block, chunk 4*slice + (l >> 4)
@@ -339,20 +345,29 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
         voff[q] = row < BM ? (uint32_t)(row * p.lda + chunk * 8) * 2u
                            : (uint32_t)((row - BM) * p.ldb + chunk * 8) * 2u;
     }
-    // (the chunk a lane fetches depends on the parity of the instruction only: swz(8 * inst + lr))
-    const bool tail_ok[2] = {(lc ^ (lr >> 1)) < tail_chunks, (lc ^ (4 | (lr >> 1))) < tail_chunks};
+    // (the chunk a lane fetches depends on the parity of the instruction only: swz(8 * inst + lr);
+    // `even` / `odd` below are the parities of q, the wave's first instruction being wave * LW)
+    const int par0 = (wave * LW) & 1;
+    const int chunk_even = lc ^ ((par0 << 2) | (lr >> 1)), chunk_odd = lc ^ (((par0 ^ 1) << 2) | (lr >> 1));
+    const bool tail_ok_even = chunk_even < tail_chunks, tail_ok_odd = chunk_odd < tail_chunks;
     // `rq_unit` follows the unit about to be requested; requests past the last unit fetch nothing
     int rq_unit = 0;
-    auto request = [&](int stage) __attribute__((always_inline)) {
+    auto request = [&](int stage, auto maybe_tail_c) __attribute__((always_inline)) {
         const bool live = rq_unit < KT;
-        const bool tail = tail_chunks != 0 && rq_unit == KT - 1;
+        const bool tail = decltype(maybe_tail_c)::value && tail_chunks != 0 && rq_unit == KT - 1;
         const uint32_t kb = (uint32_t)rq_unit * 128u;
         ++rq_unit;
         const uint32_t dst = lds_base + (uint32_t)(stage * STAGE + wave * LW * 1024);
+        if (!tail) {
 #pragma unroll
-        for (int q = 0; q < LW; ++q)
-            dma(live ? ((wave * LW + q) * 8 < BM ? rsrcA : rsrcB) : rsrcNone,
-                (tail && !tail_ok[(wave * LW + q) & 1] ? 0x80000000u : voff[q]) + kb, dst + (uint32_t)(q * 1024));
+            for (int q = 0; q < LW; ++q)
+                dma(live ? ((wave * LW + q) * 8 < BM ? rsrcA : rsrcB) : rsrcNone, voff[q] + kb, dst + (uint32_t)(q * 1024));
+        } else {                                             // (a path of its own: nothing of it in the other units' way)
+#pragma unroll
+            for (int q = 0; q < LW; ++q)
+                dma((wave * LW + q) * 8 < BM ? rsrcA : rsrcB,
+                    ((q & 1) ? tail_ok_odd : tail_ok_even) ? voff[q] + kb : 0x80000000u, dst + (uint32_t)(q * 1024));
+        }
     };
 
     // fragment read: lane holds row l & 15 of a 16-row block, chunk 4*slice + (l >> 4)
@@ -369,7 +384,7 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
         for (int j = 0; j < NI; ++j) acc[i][j] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
 #pragma unroll
-    for (int i = 0; i < NS - 1; ++i) request(i);
+    for (int i = 0; i < NS - 1; ++i) request(i, std::true_type{});
 
     // The fragments of unit u + 1 are read while unit u is multiplied (one wave per SIMD has
     // nothing else to hide the LDS latency behind), so a unit must have landed one step before
@@ -395,21 +410,31 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
         if (tail_elems != 0 && landed == KT - 1) {
 #pragma unroll
             for (int q = 0; q < LW; ++q)
-                if ((lc ^ ((((wave * LW + q) & 1) << 2) | (lr >> 1))) == tail_chunks - 1)
+                if (((q & 1) ? chunk_odd : chunk_even) == tail_chunks - 1)
                     zero_chunk_tail(lds + stage * STAGE + (wave * LW + q) * 1024 + lane * 16, tail_elems);
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         }
         ++landed;
     };
-    // one step: unit u (fragments in set CUR) is multiplied while unit u + 1 is read into the other set
-    auto step = [&](auto cur_c) __attribute__((always_inline)) {
+    // one step: unit u (fragments in set CUR) is multiplied while unit u + 1 is read into the other set.
+    // TAIL: the step may publish or request the matrix's partial last unit.  The steps that cannot
+    // are free of branches: with more than one basic block in the loop the compiler waits for
+    // every LDS read before the first MFMA, the next unit's included (1440 x 1440 x 1472: 14.0 us
+    // against 12.4).
+    auto step = [&](auto cur_c, auto tail_c) __attribute__((always_inline)) {
         constexpr int CUR = decltype(cur_c)::value;
+        constexpr bool TAIL = decltype(tail_c)::value;
         // this wave's loads of unit u + 1 have landed; after the barrier everyone's have, and
         // everyone has multiplied unit u - 1, whose stage takes the request NS - 1 units ahead
-        asm volatile("s_waitcnt vmcnt(%0)" :: "n"((NS - 3) * LW) : "memory");
-        fix_tail(s + 1 == NS ? 0 : s + 1);
-        asm volatile("s_barrier" ::: "memory");
-        request(s == 0 ? NS - 1 : s - 1);
+        if constexpr (TAIL) {
+            asm volatile("s_waitcnt vmcnt(%0)" :: "n"((NS - 3) * LW) : "memory");
+            fix_tail(s + 1 == NS ? 0 : s + 1);
+            asm volatile("s_barrier" ::: "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"((NS - 3) * LW) : "memory");
+            ++landed;
+        }
+        request(s == 0 ? NS - 1 : s - 1, tail_c);
         read_unit(s + 1 == NS ? 0 : s + 1, fa[CUR ^ 1], fb[CUR ^ 1]);   // (past the last unit: zeros or stale rows, never multiplied)
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -426,12 +451,18 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
     fix_tail(0);
     asm volatile("s_barrier" ::: "memory");
     read_unit(0, fa[0], fb[0]);
+    // the partial last unit (if any) is requested in step KT - NS and published in step KT - 2
+    const int plain_steps = (tail_chunks != 0 ? (KT > NS ? KT - NS : 0) : KT) & ~1;
     int u = 0;
-    for (; u + 2 <= KT; u += 2) {
-        step(std::integral_constant<int, 0>{});
-        step(std::integral_constant<int, 1>{});
+    for (; u < plain_steps; u += 2) {
+        step(std::integral_constant<int, 0>{}, std::false_type{});
+        step(std::integral_constant<int, 1>{}, std::false_type{});
     }
-    if (u < KT) step(std::integral_constant<int, 0>{});
+    for (; u + 2 <= KT; u += 2) {
+        step(std::integral_constant<int, 0>{}, std::true_type{});
+        step(std::integral_constant<int, 1>{}, std::true_type{});
+    }
+    if (u < KT) step(std::integral_constant<int, 0>{}, std::true_type{});
     // requests past the last unit (empty descriptor: zeros) are still heading for the ring, and
     // other waves may still be reading the last stage: drain and meet before C takes its place
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
