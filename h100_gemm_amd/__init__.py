@@ -156,6 +156,11 @@ def select_config(M: int, N: int, K: int, dtype: int = MI_DTYPE_BF16) -> int:
     return _lib.load().mi_gemm_select_config(dtype, M, N, K)
 
 
+def row_cut(M: int, N: int, K: int, dtype: int = MI_DTYPE_BF16) -> int:
+    """Rows the automatic choice runs as a GEMM of their own ahead of the rest (0: one GEMM)."""
+    return _lib.load().mi_gemm_row_cut(dtype, M, N, K)
+
+
 def config_grid(config: int, M: int, N: int, K: int) -> int:
     return _lib.load().mi_gemm_config_grid(config, M, N, K)
 

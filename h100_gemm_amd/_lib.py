@@ -54,6 +54,7 @@ SYMBOLS = {
     "mi_gemm_find_config": (C.c_int, [C.c_char_p]),
     "mi_gemm_select_config": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int]),
     "mi_gemm_tuned_entries": (C.c_int, []),
+    "mi_gemm_row_cut": (C.c_int, [C.c_int] * 4),
     "mi_gemm_config_supports": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]),
     "mi_gemm_config_grid": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int]),
     "mi_gemm_config_lds_bytes": (C.c_int, [C.c_int]),

@@ -354,12 +354,40 @@ Choice choose(int requested, int M, int N, int K, bool streamable, bool splittab
     return c;
 }
 
+// The cut of a large ragged shape into two GEMMs is a pure function of the shape and four flags
+// like the kernel choice, and costs several passes of the time model: the last answer is kept per
+// thread.  MI_GEMM_ROW_CUT=0 switches the cut off (measurement aid).
+int rows_to_cut(int M, int N, int K, bool streamable, bool splittable, bool ptr_aligned, bool small_ok) {
+    static const int env = [] { const char* s = getenv("MI_GEMM_ROW_CUT"); return s ? atoi(s) : 1; }();
+    if (env == 0 || (long long)M * N < 4096LL * 4096LL) return 0;
+    struct Memo { int M, N, K, flags, cus, m1; };
+    static thread_local Memo memo = {0, 0, 0, -1, 0, 0};
+    const int flags = (streamable ? 1 : 0) | (splittable ? 2 : 0) | (ptr_aligned ? 4 : 0) | (small_ok ? 8 : 0);
+    const int cus = compute_units();
+    if (memo.M != M || memo.N != N || memo.K != K || memo.flags != flags || memo.cus != cus)
+        memo = {M, N, K, flags, cus, mi::rows_to_split_off(M, N, K, streamable, splittable, ptr_aligned, small_ok, cus)};
+    return memo.m1;
+}
+
 // One GEMM launch (two for split-K): argument checks, kernel choice, aligned / predicated twin.
+// `may_cut`: the automatic choice may run the shape as two GEMMs, the first rows and the rest
+// (rows_to_split_off in the kernel table); the parts themselves are not cut again.
 int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const void* B, void* C,
-             int* DB, float alpha, float beta, void* stream, const WsSource& wsrc = WsSource{}) {
+             int* DB, float alpha, float beta, void* stream, const WsSource& wsrc = WsSource{}, bool may_cut = true) {
     int rc = check_args(config, dtype, M, N, K, A, B, C);
     if (rc != MI_OK) return rc;
     const bool streamable = shape_is_streamable(M, N, K, A, B, C);
+    if (may_cut && config == MI_CONFIG_AUTO && DB == nullptr &&
+        tuned_config(M, N, K, streamable, shape_has_word_rows(K, A, B)) < 0) {       // (a tuned shape runs as tuned)
+        const int m1 = rows_to_cut(M, N, K, streamable, shape_is_splittable(N, C, DB),
+                                   aligned16(A) && aligned16(B) && aligned16(C), shape_has_word_rows(K, A, B));
+        if (m1 > 0) {
+            rc = run_gemm(config, dtype, m1, N, K, A, B, C, nullptr, alpha, beta, stream, wsrc, false);
+            if (rc != MI_OK) return rc;
+            return run_gemm(config, dtype, M - m1, N, K, (const unsigned char*)A + (size_t)m1 * K * 2, B,
+                            (unsigned char*)C + (size_t)m1 * N * 2, nullptr, alpha, beta, stream, wsrc, false);
+        }
+    }
     // with a trace buffer the automatic choice stays with the kernels that fill it (the tiled
     // ones); an explicitly requested decode or small-tile kernel runs and leaves it untouched
     const Choice choice = choose(config, M, N, K, streamable && !(config == MI_CONFIG_AUTO && DB),
@@ -529,6 +557,14 @@ int mi_gemm_select_config(int dtype, int M, int N, int K) {
     return mi::select_kernel(M, N, K, streamable, N % 4 == 0, true, K % 2 == 0, compute_units());
 }
 
+int mi_gemm_row_cut(int dtype, int M, int N, int K) {
+    (void)dtype;
+    if (!shape_in_range(M, N, K)) return 0;
+    const bool streamable = N % 4 == 0 && K % 64 == 0;
+    if (tuned_config(M, N, K, streamable, K % 2 == 0) >= 0) return 0;
+    return rows_to_cut(M, N, K, streamable, N % 4 == 0, true, K % 2 == 0);
+}
+
 int mi_gemm_tuned_entries(void) { return (int)tuned_entries().size(); }
 
 size_t mi_gemm_trace_words(int M, int N, int K) {
@@ -574,17 +610,31 @@ size_t mi_gemm_workspace_bytes(int config, int dtype, int M, int N, int K, int c
         N = t;
     }
     // The choice also depends on the alignment of the pointers, unknown here: the largest
-    // need over the cases a launch can meet.
-    size_t need = 0;
-    const bool can_stream = N % 4 == 0 && K % 64 == 0;
-    for (int aligned = 0; aligned < 2; ++aligned)
-        for (int streamable = 0; streamable < (can_stream && aligned ? 2 : 1); ++streamable) {
-            // (a launch that cannot use the small-tile kernels -- operands not 4-byte aligned -- may split where
-            // one that can does not: both cases)
-            for (int small = 0; small < (K % 2 == 0 ? 2 : 1); ++small) {
-            const Choice c = compute_choice(config, M, N, K, streamable != 0, N % 4 == 0, aligned != 0, small != 0);
-            const size_t b = c.splits > 1 ? (size_t)c.splits * M * N * sizeof(float) : 0;
-            if (b > need) need = b;
+    // need over the cases a launch can meet -- and over the two parts, where the automatic
+    // choice may cut the shape's rows in two.
+    auto uncut = [&](int rows) {
+        size_t need = 0;
+        const bool can_stream = N % 4 == 0 && K % 64 == 0;
+        for (int aligned = 0; aligned < 2; ++aligned)
+            for (int streamable = 0; streamable < (can_stream && aligned ? 2 : 1); ++streamable)
+                // (a launch that cannot use the small-tile kernels -- operands not 4-byte aligned --
+                // may split where one that can does not: both cases)
+                for (int small = 0; small < (K % 2 == 0 ? 2 : 1); ++small) {
+                    const Choice c = compute_choice(config, rows, N, K, streamable != 0, N % 4 == 0, aligned != 0, small != 0);
+                    const size_t b = c.splits > 1 ? (size_t)c.splits * rows * N * sizeof(float) : 0;
+                    if (b > need) need = b;
+                }
+        return need;
+    };
+    size_t need = uncut(M);
+    if (config == MI_CONFIG_AUTO && tuned_config(M, N, K, N % 4 == 0 && K % 64 == 0, K % 2 == 0) < 0)
+        for (int flags = 0; flags < 16; ++flags) {
+            const int m1 = rows_to_cut(M, N, K, (flags & 1) != 0 && N % 4 == 0 && K % 64 == 0, (flags & 2) != 0 && N % 4 == 0,
+                                       (flags & 4) != 0, (flags & 8) != 0 && K % 2 == 0);
+            if (m1 > 0) {
+                const size_t a = uncut(m1), b = uncut(M - m1);
+                if (a > need) need = a;
+                if (b > need) need = b;
             }
         }
     return need;

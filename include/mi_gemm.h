@@ -131,6 +131,15 @@ int mi_gemm_find_config(const char* name);
 /* The config MI_CONFIG_AUTO resolves to for this shape; -1 for a shape no launch accepts
  * (an extent <= 0, or a matrix of more than 2^31-1 elements). */
 int mi_gemm_select_config(int dtype, int M, int N, int K);
+/* Rows that MI_CONFIG_AUTO runs as a GEMM of their own ahead of the rest of the shape, or 0 (the
+ * usual case: one GEMM).  A large shape whose last row of tiles is nearly empty (7000^3 on
+ * 256x256 tiles: three rounds of workgroups and a sixteenth) is cut behind its last full row of
+ * tiles when the library's time model prices the two parts 5 % below the whole; the parts run
+ * back to back on the caller's stream, the same answers either way.  mi_gemm_select_config
+ * names the configuration the uncut shape would run.  Assumes 16-byte aligned pointers.  The
+ * reference, whose kernels take multiples of their tile only (matmul_utils.cuh:362), has no
+ * counterpart. */
+int mi_gemm_row_cut(int dtype, int M, int N, int K);
 /* Number of `M N K config-name` lines loaded from the file named by the environment variable
  * MI_GEMM_TUNED_FILE (read once, on first use; 0 without it).  MI_CONFIG_AUTO takes a listed
  * shape's configuration instead of asking the time model -- the run-time counterpart of the

@@ -429,6 +429,27 @@ def test_random_shapes_small_tile_and_decode_kinds(mi, orc):
         assert (guard == 0xEEEE).all(), "bytes outside C were written"
 
 
+def test_large_ragged_shape_cut_into_two_gemms(mi, orc):
+    """7000 x 7000 x 4096 runs as 6912 rows and then 88 (the last row of 256x256 tiles would be a
+    third full and cost a whole round): every element against the on-device golden, bit for bit
+    on an integer fill, with alpha / beta and a column-major C as well."""
+    M, N, K = 7000, 7000, 4096
+    assert mi.row_cut(M, N, K) == 6912
+    A, B = make_inputs(orc, M, N, K, "int")
+    dA, dB = mi.DeviceBuffer.from_numpy(A), mi.DeviceBuffer.from_numpy(B)
+    dC, dR = mi.DeviceBuffer(M * N * 2), mi.DeviceBuffer(M * N * 2)
+    for alpha, beta, layout in [(1.0, 0.0, mi.MI_C_ROW_MAJOR), (-0.5, 2.75, mi.MI_C_ROW_MAJOR), (1.0, 0.0, mi.MI_C_COL_MAJOR)]:
+        dC.fill_bytes(0xEE)
+        mi.gemm_epilogue(mi.GemmParams(M, N, K, dA, dB, dC, alpha=alpha, beta=beta), c_layout=layout)
+        mi.reference_gpu_gemm(mi.GemmParams(M, N, K, dA, dB, dR, alpha=alpha, beta=beta))
+        mi.synchronize()
+        C, R = dC.to_numpy((M * N,), np.uint16), dR.to_numpy((M, N), np.uint16)
+        C = C.reshape(N, M).T if layout == mi.MI_C_COL_MAJOR else C.reshape(M, N)
+        assert (C == R).all(), f"alpha {alpha} beta {beta} layout {layout}: {int((C != R).sum())} elements differ"
+    for b in (dA, dB, dC, dR):
+        b.free()
+
+
 def test_non_default_streams_and_host_threads(mi, orc):
     """The ABI's stream argument: two host threads, each launching on a stream of its own
     (created with default priority) and waiting with mi_stream_sync.  The shapes include

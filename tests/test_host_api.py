@@ -206,6 +206,14 @@ def test_config_table(mi):
     assert kc.CONFIGS[mi.select_config(512, 512, 521)]['KIND'] == 'mfma16'
     assert kc.CONFIGS[mi.select_config(512, 512, 522)]['KIND'] == 'wavek'      # rows of whole 32-bit words are enough for the small-tile kernels
     assert all("EFF" in kc.CONFIGS[mi.select_config(M, N, 4101)] for M in (257, 1000, 5000) for N in (100, 3000))
+    # a large ragged shape whose last row of tiles is nearly empty runs as two GEMMs: the rows up to
+    # the last full row of tiles, then the rest; shapes that fill their rounds, small ones and
+    # tuned ones run whole
+    assert mi.row_cut(7000, 7000, 7000) == 6912 and mi.row_cut(7000, 7000, 4096) == 6912
+    for M, N, K in [(8192, 8192, 8192), (6000, 6000, 6000), (5000, 8192, 4096), (4095, 6143, 3073), (1000, 1000, 1000),
+                    (8192, 8192, 28672), (0, 8, 8)]:
+        assert mi.row_cut(M, N, K) == 0, (M, N, K)
+    assert mi.workspace_bytes(7000, 7000, 7000) >= mi.workspace_bytes(88, 7000, 7000, config=mi.select_config(88, 7000, 7000))
     # few tiles and a long K: split-K pieces of a tiled kernel fill the CUs
     c = mi.select_config(256, 8192, 8192)
     assert kc.CONFIGS[c]["KIND"] == "mfma16" and (kc.CONFIGS[c]["BM"], kc.CONFIGS[c]["BN"]) == (256, 128)
