@@ -35,8 +35,7 @@ template takes (matmul_h100.cu.jinja:9-14) -- re-cast for CDNA4:
     WK       (wavek, optional) time model in microseconds, (fixed, per round, per unit, per
              tile): fixed + rounds of co-resident workgroups (tiles / (CUs x OCC), rounded up)
              x per round + tiles per CU (rounded up) x (per tile + K/64 x per unit);
-             non-negative least squares on 89 shapes (the 96x64 shared-ring config: x 1.07, its
-             fit being the loosest); configs that carry it join the automatic choice
+             non-negative least squares on 89-99 shapes (the 96x64 shared-ring config: x 1.035); configs that carry it join the automatic choice
     EFF_E    (optional) throughput of the predicated variant relative to the aligned one, from
              7000^3, 6000^3 and 5000^3 (default 0.85); used for shapes the aligned variant cannot run
 
@@ -276,10 +275,10 @@ CONFIGS = [
     _k(64, 64, NS=1, OCC=2, WK=(1.93, 2.19, 0.1792, 0.0)),
     _k(64, 64, NS=2, WK=(0.88, 2.81, 0.1648, 0.0)),
     _k(96, 64, NS=2, WK=(1.35, 4.06, 0.2306, 0.0)),
-    _k(96, 96, NS=4, SHARED=1, WK=(1.23, 2.555, 0.3643, 0.0), WK_RAGGED=1.18),
-    _k(64, 64, NS=4, SHARED=1, OCC=2, WK=(1.94, 1.270, 0.1847, 0.0)),
-    _k(96, 64, NS=4, SHARED=1, OCC=2, WK=(2.58, 1.43, 0.2584, 0.0)),
-    _k(64, 32, NS=4, SHARED=1, OCC=3, WK=(1.99, 0.958, 0.1252, 0.0)),
+    _k(96, 96, NS=4, SHARED=1, WK=(1.03, 3.336, 0.3179, 0.0), WK_RAGGED=1.18),
+    _k(64, 64, NS=4, SHARED=1, OCC=2, WK=(1.31, 1.734, 0.1815, 0.0)),
+    _k(96, 64, NS=4, SHARED=1, OCC=2, WK=(1.96, 1.90, 0.2313, 0.217)),
+    _k(64, 32, NS=4, SHARED=1, OCC=3, WK=(1.54, 1.362, 0.1234, 0.0)),
 ]
 
 assert all(is_valid_config(c) for c in CONFIGS), [config_name(c) for c in CONFIGS if not is_valid_config(c)]
