@@ -189,7 +189,8 @@ def test_config_table(mi):
     for M, N, K in [(1440, 1440, 1472), (1344, 1344, 1344), (1536, 1472, 320)]:
         c = kc.CONFIGS[mi.select_config(M, N, K)]
         assert c["KIND"] == "wavek" and c.get("SHARED") == 1, (M, N, K, c)
-    assert mi.config_name(mi.select_config(1536, 1536, 1536)) == "m128x128_w2x2_g4_b1_k2"
+    assert mi.config_name(mi.select_config(1536, 1536, 1536)) == "k96x96_s4"               # 256 tiles of 96x96, one per CU
+    assert mi.config_name(mi.select_config(2048, 2048, 2048)) == "m128x128_w2x2_g4_b1_k2"  # 256 tiles of 128x128, two K groups each
     # wave quantisation: 256 CUs; 8192^2 fills four rounds of 256x256 tiles, 4095x6143 fills
     # two rounds of 256x192 tiles exactly (256x256 would leave half of the second round
     # idle), and 512^2 is a single partial round whatever the tiled kernel: the small-tile
