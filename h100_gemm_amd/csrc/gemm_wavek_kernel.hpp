@@ -43,9 +43,9 @@
 // single stage and one workgroup per CU only, were far behind the tiled kernels (2048^3:
 // 26.5 us against 19.6): alone and with one stage, loading and multiplying take turns.
 // Rows of A past M and rows of B past N are never fetched (the buffer descriptors end at the
-// last valid row of the tile).  Preconditions, checked by the launcher's caller: K even and
-// 4-byte aligned A and B (rows of whole 32-bit words, which is what the descriptors' range check
-// counts in; a partial last unit of K is filled up with zeros).  Any N and any C: where the
+// last valid row of the tile).  Precondition, checked by the launcher's caller: 4-byte aligned A
+// and B.  Any K (a partial last unit is filled up with zeros; the last k of an odd K is added in
+// the epilogue).  Any N and any C: where the
 // groups of four elements do not all start on 8-byte boundaries inside N, C is stored element
 // by element.  Rows that start on 128-byte boundaries (K % 64 == 0, aligned bases) are what the
 // kernel is fastest on: with any other pitch every 128-byte piece of a row straddles two lines.
@@ -71,6 +71,14 @@ __device__ __forceinline__ void zero_chunk_tail(unsigned char* ptr, int keep_ele
 #pragma unroll
     for (int w = 0; w < 4; ++w) v[w] = w < keep_words ? v[w] : 0u;
     *(u32x4_t*)ptr = v;
+}
+
+// One element of A or B as fp32 (the last k of an odd K, which the loops below leave out).
+template <int DT>
+__device__ __forceinline__ float load_elem(const void* base, size_t index) {
+    const uint16_t u = ((const uint16_t*)base)[index];
+    if constexpr (DT == DT_BF16) return __builtin_bit_cast(float, (uint32_t)u << 16);
+    else return (float)__builtin_bit_cast(_Float16, u);
 }
 
 template <int BM_, int BN_, int NS_, int DT_>
@@ -108,9 +116,13 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
     int tm, tn;
     tile_of_block<4>(blockIdx.x, gridDim.x, tiles_m, tiles_n, tm, tn);
     const int row0 = tm * BM, col0 = tn * BN;
-    const int KT = (K + 63) / 64;                            // units of K; the last may be partial (K even)
-    const int tail_chunks = ((K & 63) + 7) >> 3;             // 16-byte chunks of a row in a partial last unit (0: none)
-    const int tail_elems = K & 7;                            // elements of k < K in the last of them (0: all eight)
+    // An odd K: the loops take the even part, whole 32-bit words of every row (so that no word the
+    // descriptors' range check passes or drops is half inside a row), and the last k is added to
+    // the sums in the epilogue, one product per element.
+    const int Ke = K & ~1;
+    const int KT = (Ke + 63) / 64;                           // units of K; the last may be partial
+    const int tail_chunks = ((Ke & 63) + 7) >> 3;            // 16-byte chunks of a row in a partial last unit (0: none)
+    const int tail_elems = Ke & 7;                           // elements of k < Ke in the last of them (0: all eight)
     const int cnt = (KT - wave + 3) / 4;                     // units of this wave: wave, wave+4, ...
 
     const int rowsA = (M - row0) < BM ? (M - row0) : BM;
@@ -242,6 +254,12 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
             const f32x4_t v = *(const f32x4_t*)((const float*)(lds + w * REGION) + m * PITCH + n);
             sum[0] += v[0]; sum[1] += v[1]; sum[2] += v[2]; sum[3] += v[3];
         }
+        if ((K & 1) != 0 && row0 + m < M) {                  // the last k of an odd K
+            const float a_last = load_elem<DT>(p.A, (size_t)(row0 + m) * p.lda + K - 1);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (col0 + n + e < N) sum[e] += a_last * load_elem<DT>(p.B, (size_t)(col0 + n + e) * p.ldb + K - 1);
+        }
         if (scaled) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) sum[e] = mul_add_unfused(sum[e], p.alpha, p.beta);
@@ -312,9 +330,13 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
     int tm, tn;
     tile_of_block<4>(blockIdx.x, gridDim.x, tiles_m, tiles_n, tm, tn);
     const int row0 = tm * BM, col0 = tn * BN;
-    const int KT = (K + 63) / 64;                            // units of K; the last may be partial (K even)
-    const int tail_chunks = ((K & 63) + 7) >> 3;             // 16-byte chunks of a row in a partial last unit (0: none)
-    const int tail_elems = K & 7;                            // elements of k < K in the last of them (0: all eight)
+    // An odd K: the loops take the even part, whole 32-bit words of every row (so that no word the
+    // descriptors' range check passes or drops is half inside a row), and the last k is added to
+    // the sums in the epilogue, one product per element.
+    const int Ke = K & ~1;
+    const int KT = (Ke + 63) / 64;                           // units of K; the last may be partial
+    const int tail_chunks = ((Ke & 63) + 7) >> 3;            // 16-byte chunks of a row in a partial last unit (0: none)
+    const int tail_elems = Ke & 7;                           // elements of k < Ke in the last of them (0: all eight)
 
     const int rowsA = (M - row0) < BM ? (M - row0) : BM;
     const int rowsB = (N - col0) < BN ? (N - col0) : BN;
@@ -488,6 +510,12 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
         const int q = it * 256 + tid;
         const int m = q / (BN / 4), n = (q % (BN / 4)) * 4;
         f32x4_t sum = *(const f32x4_t*)(part + m * PITCH + n);
+        if ((K & 1) != 0 && row0 + m < M) {                  // the last k of an odd K
+            const float a_last = load_elem<DT>(p.A, (size_t)(row0 + m) * p.lda + K - 1);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (col0 + n + e < N) sum[e] += a_last * load_elem<DT>(p.B, (size_t)(col0 + n + e) * p.ldb + K - 1);
+        }
         if (scaled) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) sum[e] = mul_add_unfused(sum[e], p.alpha, p.beta);

@@ -55,11 +55,11 @@ bool shape_is_streamable(int M, int N, int K, const void* A, const void* B, cons
     return N % 4 == 0 && K % 64 == 0 && aligned16(A) && aligned16(B) &&
            (((uintptr_t)C & 7u) == 0);
 }
-// The small-tile kernels fill a partial last K unit with zeros and store a C of any N and
-// alignment: rows of A and B made of whole 32-bit words (K even, 4-byte aligned bases) are all
-// they need.
+// The small-tile kernels take any M, N and K and store a C of any alignment: A and B on 4-byte
+// boundaries are all they need.
 bool shape_has_word_rows(int K, const void* A, const void* B) {
-    return K % 2 == 0 && (((uintptr_t)A | (uintptr_t)B) & 3u) == 0;
+    (void)K;
+    return (((uintptr_t)A | (uintptr_t)B) & 3u) == 0;
 }
 
 // Split-K geometry for a decode launch.  The decode kernel is bound by what one CU can pull
@@ -429,7 +429,7 @@ int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const vo
     }
     if (e.kind == mi::KIND_WAVEK) {
         if (!shape_has_word_rows(K, A, B))
-            return fail(MI_ERR_UNSUPPORTED, "config %s needs an even K and 4-byte aligned A and B", e.name);
+            return fail(MI_ERR_UNSUPPORTED, "config %s needs 4-byte aligned A and B", e.name);
         hipError_t err = e.launch[dtype][0](args, (hipStream_t)stream);
         if (err != hipSuccess)
             return fail(MI_ERR_HIP, "launch of %s failed: %s", e.name, hipGetErrorString(err));
@@ -524,7 +524,7 @@ int mi_gemm_config_supports(int config, int dtype, int M, int N, int K) {
     const mi::KernelEntry& e = mi::kKernels[config];
     if (is_split_k_decode(e.kind) || e.kind == mi::KIND_STREAM)
         return M <= e.BM && N % 4 == 0 && K % 64 == 0;
-    if (e.kind == mi::KIND_WAVEK) return K % 2 == 0;
+    if (e.kind == mi::KIND_WAVEK) return 1;
     if (e.kg > 1 && K % (128 * e.kg) != 0) return 0;
     return e.launch[dtype][1] != nullptr;
 }
@@ -539,7 +539,7 @@ int mi_gemm_config_grid(int config, int M, int N, int K) {
         return tiles_n * choose_splits(tiles_n, K, compute_units());
     }
     const int tiles = ((M + e.BM - 1) / e.BM) * ((N + e.BN - 1) / e.BN);
-    if (e.kind == mi::KIND_WAVEK) return K % 2 != 0 ? 0 : tiles;
+    if (e.kind == mi::KIND_WAVEK) return tiles;
     if (e.kind == mi::KIND_MFMA16) {   // split-K pieces, assuming an aligned C and no trace buffer
         int kps = K;
         return tiles * choose_tile_splits(e, M, N, K, N % 4 == 0, true, compute_units(), &kps);
@@ -552,17 +552,17 @@ int mi_gemm_select_config(int dtype, int M, int N, int K) {
     if (!shape_in_range(M, N, K)) return -1;
     // pointer alignment is unknown here: assume the usual 256-byte aligned allocations
     const bool streamable = N % 4 == 0 && K % 64 == 0;
-    const int tuned = tuned_config(M, N, K, streamable, K % 2 == 0);
+    const int tuned = tuned_config(M, N, K, streamable, true);
     if (tuned >= 0) return tuned;
-    return mi::select_kernel(M, N, K, streamable, N % 4 == 0, true, K % 2 == 0, compute_units());
+    return mi::select_kernel(M, N, K, streamable, N % 4 == 0, true, true, compute_units());
 }
 
 int mi_gemm_row_cut(int dtype, int M, int N, int K) {
     (void)dtype;
     if (!shape_in_range(M, N, K)) return 0;
     const bool streamable = N % 4 == 0 && K % 64 == 0;
-    if (tuned_config(M, N, K, streamable, K % 2 == 0) >= 0) return 0;
-    return rows_to_cut(M, N, K, streamable, N % 4 == 0, true, K % 2 == 0);
+    if (tuned_config(M, N, K, streamable, true) >= 0) return 0;
+    return rows_to_cut(M, N, K, streamable, N % 4 == 0, true, true);
 }
 
 int mi_gemm_tuned_entries(void) { return (int)tuned_entries().size(); }
@@ -619,7 +619,7 @@ size_t mi_gemm_workspace_bytes(int config, int dtype, int M, int N, int K, int c
             for (int streamable = 0; streamable < (can_stream && aligned ? 2 : 1); ++streamable)
                 // (a launch that cannot use the small-tile kernels -- operands not 4-byte aligned --
                 // may split where one that can does not: both cases)
-                for (int small = 0; small < (K % 2 == 0 ? 2 : 1); ++small) {
+                for (int small = 0; small < 2; ++small) {
                     const Choice c = compute_choice(config, rows, N, K, streamable != 0, N % 4 == 0, aligned != 0, small != 0);
                     const size_t b = c.splits > 1 ? (size_t)c.splits * rows * N * sizeof(float) : 0;
                     if (b > need) need = b;
@@ -627,10 +627,10 @@ size_t mi_gemm_workspace_bytes(int config, int dtype, int M, int N, int K, int c
         return need;
     };
     size_t need = uncut(M);
-    if (config == MI_CONFIG_AUTO && tuned_config(M, N, K, N % 4 == 0 && K % 64 == 0, K % 2 == 0) < 0)
+    if (config == MI_CONFIG_AUTO && tuned_config(M, N, K, N % 4 == 0 && K % 64 == 0, true) < 0)
         for (int flags = 0; flags < 16; ++flags) {
             const int m1 = rows_to_cut(M, N, K, (flags & 1) != 0 && N % 4 == 0 && K % 64 == 0, (flags & 2) != 0 && N % 4 == 0,
-                                       (flags & 4) != 0, (flags & 8) != 0 && K % 2 == 0);
+                                       (flags & 4) != 0, (flags & 8) != 0);
             if (m1 > 0) {
                 const size_t a = uncut(m1), b = uncut(M - m1);
                 if (a > need) need = a;

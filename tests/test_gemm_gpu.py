@@ -226,10 +226,17 @@ def test_wave_split_k_kernels(mi, orc, config):
     check_epilogue(mi, orc, 300, 260, 1000, "int", -0.5, 2.75, config=config, exact=True)
     check_epilogue(mi, orc, 300, 261, 1002, "int", -0.5, 2.75, config=config, exact=True)
     check_epilogue(mi, orc, 200, 131, 1026, "int", 2.0, -1.0, config=config, c_layout=mi.MI_C_COL_MAJOR, exact=True)
-    for M, N, K in [(256, 256, 101), (256, 254, 1)]:
-        A, B = make_inputs(orc, M, N, K, "int")
+    # an odd K: the loops take the even part, the last k is added in the epilogue
+    for M, N, K in [(bm, bn, 1), (bm + 3, bn + 1, 3), (97, 101, 65), (300, 259, 101), (500, 500, 501),
+                    (257, 515, 77), (1001, 1001, 1001), (130, 130, 191), (7, 3, 255), (640, 77, 4101)]:
+        check(mi, orc, M, N, K, "int", config=config, exact=True)
+    check(mi, orc, 999, 1001, 1003, "uniform", config=config)
+    check(mi, orc, 300, 201, 501, "normal", config=config, dtype=orc.FP16)
+    check_epilogue(mi, orc, 300, 261, 1003, "int", -0.5, 2.75, config=config, exact=True)
+    # operands that do not start on 4-byte boundaries are refused, not mis-computed
+    for offA, offB in [(2, 0), (0, 6)]:
         with pytest.raises(mi.MiGemmError) as ei:
-            Dev(mi, A, B, M, N).run(K, config=config)
+            _run_offset(mi, orc, config, 100, 100, 128, offA, offB, 0)
         assert ei.value.code == mi._lib.MI_ERR_UNSUPPORTED
 
 
@@ -413,9 +420,9 @@ def test_random_shapes_small_tile_and_decode_kinds(mi, orc):
         offA, offB, offC = 16 * int(rng.integers(0, 4)), 16 * int(rng.integers(0, 4)), 8 * int(rng.integers(0, 8))
         pool = special
         if it % 2 == 1:
-            # what only the small-tile kernels take: any even K, any N, operands on 4-byte and C on
+            # what only the small-tile kernels take: any K, any N, operands on 4-byte and C on
             # 2-byte boundaries
-            K = 2 * int(rng.choice([rng.integers(1, 40), rng.integers(40, 1300)]))
+            K = int(rng.choice([rng.integers(1, 80), rng.integers(80, 2600)]))
             N = int(rng.integers(1, 720))
             offA, offB, offC = 4 * int(rng.integers(0, 16)), 4 * int(rng.integers(0, 16)), 2 * int(rng.integers(0, 32))
             pool = small

@@ -146,12 +146,12 @@ def test_config_table(mi):
             assert mi.config_grid(i, 16, 8192, 8192) >= 64
             assert mi.config_grid(i, c["BM"] + 1, 8192, 8192) == 0
         elif c["KIND"] == "wavek":
-            # any M and N; rows of whole 32-bit words (an even K); no ragged twin
+            # any M, N and K (operands on 4-byte boundaries, which a shape does not tell); no ragged twin
             assert mi.config_grid(i, 1000, 780, 64) == -(-1000 // c["BM"]) * -(-780 // c["BN"])
             assert L.mi_gemm_config_supports(i, 0, 1000, 780, 4096) == 1
             assert L.mi_gemm_config_supports(i, 0, 1000, 777, 4098) == 1
-            assert L.mi_gemm_config_supports(i, 0, 1000, 780, 4097) == 0
-            assert mi.config_grid(i, 1000, 780, 4097) == 0
+            assert L.mi_gemm_config_supports(i, 0, 1, 1, 1) == 1
+            assert mi.config_grid(i, 1000, 780, 4097) == mi.config_grid(i, 1000, 780, 64)
         elif c.get("KG", 1) > 1:
             # K split over groups of waves inside the workgroup: any M, N; K in equal halves of whole double steps
             assert L.mi_gemm_config_supports(i, 0, 4095, 6143, 3072) == 1
@@ -180,9 +180,9 @@ def test_config_table(mi):
     # few tiles and a long K: small tiles with K split over the waves, when the kernel can run the shape
     assert kc.CONFIGS[mi.select_config(512, 512, 4096)]["KIND"] == "wavek"
     assert kc.CONFIGS[mi.select_config(1024, 1024, 4096)]["KIND"] == "wavek"
-    assert kc.CONFIGS[mi.select_config(512, 512, 4100)]["KIND"] == "wavek"     # an even K and any N will do
+    assert kc.CONFIGS[mi.select_config(512, 512, 4100)]["KIND"] == "wavek"     # any K and any N will do
     assert kc.CONFIGS[mi.select_config(512, 510, 4096)]["KIND"] == "wavek"
-    assert kc.CONFIGS[mi.select_config(512, 512, 4101)]["KIND"] == "mfma16"    # an odd K: the predicated tiled kernels
+    assert kc.CONFIGS[mi.select_config(512, 511, 4101)]["KIND"] == "wavek"
     # a mid-sized output with a K of moderate length: small tiles on a shared ring (K is not split
     # over the waves), also with a short K and many tiles, where the K-splitting ones are shut out
     assert not kc.CONFIGS[mi.select_config(512, 512, 4096)].get("SHARED")
@@ -194,7 +194,7 @@ def test_config_table(mi):
     # wave quantisation: 256 CUs; 8192^2 fills four rounds of 256x256 tiles, 4095x6143 fills
     # two rounds of 256x192 tiles exactly (256x256 would leave half of the second round
     # idle), and 512^2 is a single partial round whatever the tiled kernel: the small-tile
-    # kernel gives every CU a 32x32 tile (one with an odd K cannot run it: 128x128 tiles)
+    # kernel gives every CU a 32x32 tile
     def picked(M, N, K):
         c = kc.CONFIGS[mi.select_config(M, N, K)]
         return c["BM"], c["BN"]
@@ -203,10 +203,8 @@ def test_config_table(mi):
     assert picked(4095, 6143, 3073) == (256, 192)
     assert picked(512, 512, 512) == (32, 32)
     assert kc.CONFIGS[mi.select_config(512, 512, 512)]['KIND'] == 'wavek'
-    assert picked(512, 512, 521) == (128, 128)
-    assert kc.CONFIGS[mi.select_config(512, 512, 521)]['KIND'] == 'mfma16'
-    assert kc.CONFIGS[mi.select_config(512, 512, 522)]['KIND'] == 'wavek'      # rows of whole 32-bit words are enough for the small-tile kernels
-    assert all("EFF" in kc.CONFIGS[mi.select_config(M, N, 4101)] for M in (257, 1000, 5000) for N in (100, 3000))
+    assert kc.CONFIGS[mi.select_config(512, 512, 521)]['KIND'] == 'wavek'      # a ragged K too
+    assert all("EFF" in kc.CONFIGS[mi.select_config(M, N, 4101)] for M in (3000, 5000) for N in (3000, 6001))   # large: tiled
     # a large ragged shape whose last row of tiles is nearly empty runs as two GEMMs: the rows up to
     # the last full row of tiles, then the rest; shapes that fill their rounds, small ones and
     # tuned ones run whole
@@ -222,7 +220,8 @@ def test_config_table(mi):
     c = mi.find_config("m128x128_w2x2_g4_b1_o2")                    # (the automatic choice is the small-tile kernel)
     assert mi.config_grid(c, 512, 512, 4096) == 16 * 8              # 128x128 tiles x 8 pieces of 512
     assert mi.config_grid(mi.select_config(8192, 8192, 8192), 8192, 8192, 8192) == 1024   # no split-K when the tiles fill the chip
-    assert mi.config_grid(mi.select_config(512, 512, 521), 512, 512, 521) == 16           # nor for a short K
+    c = mi.find_config("m128x128_w2x2_g4_b1_o2")
+    assert mi.config_grid(c, 512, 512, 521) == 16                                         # nor for a short K
     assert mi.config_grid(mi.select_config(512, 512, 512), 512, 512, 512) == 256          # 32x32 tiles, one per CU
     c = mi.select_config(512, 510, 4097)
     assert mi.config_grid(c, 512, 510, 4097) == -(-512 // kc.CONFIGS[c]["BM"]) * -(-510 // kc.CONFIGS[c]["BN"])   # N % 4 != 0: no split-K
