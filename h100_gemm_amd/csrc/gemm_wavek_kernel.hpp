@@ -90,13 +90,15 @@ struct WaveKConfig {
     static constexpr int STAGE = (BM + BN) * 128;            // bytes of a ring stage
     static constexpr int RING = NS * STAGE;
     static constexpr int PITCH = BN + 4;                     // floats per row of a partial tile (bank spread)
-    static constexpr int PART = BM * PITCH * 4;
+    static constexpr int TILE = BM * PITCH * 4;              // bytes of a tile of fp32 sums
+    static constexpr int PART = TILE + (BM + BN) * 4;         // ... and, behind it, the last k of an odd K: A[row0 + m][K-1], then B[col0 + n][K-1]
     static constexpr int REGION = RING > PART ? RING : PART; // one wave's share of LDS
     static constexpr int LDS_BYTES = NW * REGION;
     static constexpr int QUADS = BM * BN / 4 / NT;           // 4-element groups of C per thread
     static_assert(BM % 16 == 0 && BN % 16 == 0, "whole 16x16 MFMA tiles");
     static_assert(NS >= 1 && (NS - 1) * L <= 63, "vmcnt is a 6-bit counter");
     static_assert(BM * BN / 4 % NT == 0, "the C tile divides over the threads");
+    static_assert(BM + BN <= NT, "one thread per row of the A and B panels fetches the last k of an odd K");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
 };
 
@@ -123,6 +125,15 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
     const int KT = (Ke + 63) / 64;                           // units of K; the last may be partial
     const int tail_chunks = ((Ke & 63) + 7) >> 3;            // 16-byte chunks of a row in a partial last unit (0: none)
     const int tail_elems = Ke & 7;                           // elements of k < Ke in the last of them (0: all eight)
+    // the last k of an odd K: one element per row of the A and B panels, asked for now, put into
+    // LDS after the loops (rows outside M or N count as zero)
+    float last_elem = 0.0f;
+    if ((K & 1) != 0 && tid < BM + BN) {
+        const bool of_a = tid < BM;
+        const int r = of_a ? row0 + tid : col0 + tid - BM;
+        if (r < (of_a ? M : N))
+            last_elem = load_elem<DT>(of_a ? p.A : p.B, (size_t)r * (of_a ? p.lda : p.ldb) + K - 1);
+    }
     const int cnt = (KT - wave + 3) / 4;                     // units of this wave: wave, wave+4, ...
 
     const int rowsA = (M - row0) < BM ? (M - row0) : BM;
@@ -236,6 +247,10 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
     // ---- add the four partial tiles in wave order, scale, round, store ----
     // acc[i][j][e] of lane l is P[m][n], m = i*16 + (l & 15), n = j*16 + 4*(l >> 4) + e
     float* part = (float*)(lds + wave * REGION);
+    // entry t of the last-k row (fetched by thread t) sits behind the tile of wave t / 64, which
+    // that wave is done with; the other waves may still be in their loops
+    auto last_k = [&](int t) { return (float*)(lds + (t >> 6) * REGION + Cfg::TILE) + (t & 63); };
+    if (tid < BM + BN) *last_k(tid) = last_elem;
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
@@ -254,11 +269,11 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
             const f32x4_t v = *(const f32x4_t*)((const float*)(lds + w * REGION) + m * PITCH + n);
             sum[0] += v[0]; sum[1] += v[1]; sum[2] += v[2]; sum[3] += v[3];
         }
-        if ((K & 1) != 0 && row0 + m < M) {                  // the last k of an odd K
-            const float a_last = load_elem<DT>(p.A, (size_t)(row0 + m) * p.lda + K - 1);
+        if ((K & 1) != 0) {                                  // the last k of an odd K
+            const float a_last = *last_k(m);
+            const f32x4_t b_last = *(const f32x4_t*)last_k(BM + n);
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (col0 + n + e < N) sum[e] += a_last * load_elem<DT>(p.B, (size_t)(col0 + n + e) * p.ldb + K - 1);
+            for (int e = 0; e < 4; ++e) sum[e] += a_last * b_last[e];
         }
         if (scaled) {
 #pragma unroll
@@ -303,13 +318,15 @@ struct SharedRingConfig {
     static constexpr int STAGE = (BM + BN) * 128;
     static constexpr int RING = NS * STAGE;
     static constexpr int PITCH = BN + 4;                     // floats per row of the staged C tile (bank spread)
-    static constexpr int PART = BM * PITCH * 4;
+    static constexpr int TILE = BM * PITCH * 4;              // bytes of a tile of fp32 sums
+    static constexpr int PART = TILE + (BM + BN) * 4;         // ... and, behind it, the last k of an odd K: A[row0 + m][K-1], then B[col0 + n][K-1]
     static constexpr int LDS_BYTES = RING > PART ? RING : PART;
     static constexpr int QUADS = BM * BN / 4 / NT;           // 4-element groups of C per thread
     static_assert(BM % 32 == 0 && BN % 32 == 0, "wave tiles of whole 16x16 MFMA tiles");
     static_assert(L % NW == 0, "a stage's load instructions divide over the waves");
     static_assert(NS >= 3 && (NS - 1) * LW <= 63, "a unit being read, one being multiplied, the rest in flight; vmcnt is a 6-bit counter");
     static_assert(BM * BN / 4 % NT == 0, "the C tile divides over the threads");
+    static_assert(BM + BN <= NT, "one thread per row of the A and B panels fetches the last k of an odd K");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
 };
 
@@ -337,6 +354,15 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
     const int KT = (Ke + 63) / 64;                           // units of K; the last may be partial
     const int tail_chunks = ((Ke & 63) + 7) >> 3;            // 16-byte chunks of a row in a partial last unit (0: none)
     const int tail_elems = Ke & 7;                           // elements of k < Ke in the last of them (0: all eight)
+    // the last k of an odd K: one element per row of the A and B panels, asked for now, put into
+    // LDS after the loops (rows outside M or N count as zero)
+    float last_elem = 0.0f;
+    if ((K & 1) != 0 && tid < BM + BN) {
+        const bool of_a = tid < BM;
+        const int r = of_a ? row0 + tid : col0 + tid - BM;
+        if (r < (of_a ? M : N))
+            last_elem = load_elem<DT>(of_a ? p.A : p.B, (size_t)r * (of_a ? p.lda : p.ldb) + K - 1);
+    }
 
     const int rowsA = (M - row0) < BM ? (M - row0) : BM;
     const int rowsB = (N - col0) < BN ? (N - col0) : BN;
@@ -497,6 +523,8 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
     // ---- the C tile through LDS as fp32, then scaled, rounded once and stored 8 bytes per lane ----
     // acc[i][j][e] of lane l is C[m][n], m = wm*TM + i*16 + (l & 15), n = wn*TN + j*16 + 4*(l >> 4) + e
     float* part = (float*)lds;
+    float* last_k = (float*)(lds + Cfg::TILE);
+    if (tid < BM + BN) last_k[tid] = last_elem;
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
@@ -510,11 +538,11 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
         const int q = it * 256 + tid;
         const int m = q / (BN / 4), n = (q % (BN / 4)) * 4;
         f32x4_t sum = *(const f32x4_t*)(part + m * PITCH + n);
-        if ((K & 1) != 0 && row0 + m < M) {                  // the last k of an odd K
-            const float a_last = load_elem<DT>(p.A, (size_t)(row0 + m) * p.lda + K - 1);
+        if ((K & 1) != 0) {                                  // the last k of an odd K
+            const float a_last = last_k[m];
+            const f32x4_t b_last = *(const f32x4_t*)(last_k + BM + n);
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (col0 + n + e < N) sum[e] += a_last * load_elem<DT>(p.B, (size_t)(col0 + n + e) * p.ldb + K - 1);
+            for (int e = 0; e < 4; ++e) sum[e] += a_last * b_last[e];
         }
         if (scaled) {
 #pragma unroll
