@@ -17,7 +17,7 @@ template takes (matmul_h100.cu.jinja:9-14) -- re-cast for CDNA4:
              shapes, M <= BM, whose LDS ring holds B only, csrc/gemm_decode_kernel.hpp) or
              "stream" (single-pass decode kernel, csrc/gemm_stream_kernel.hpp), "wavek" (small
              tiles with K split over the waves of a workgroup, or on a ring shared by them, for
-             outputs of few tiles: any M and N, any even K, csrc/gemm_wavek_kernel.hpp)
+             outputs of few tiles: any M, N and K, csrc/gemm_wavek_kernel.hpp)
     EPI      1: C tile transposed through LDS and written 16 bytes per lane, 0: 8-byte stores
     KG       (mfma16, optional) 2: eight waves as two groups that each multiply half of K of the
              same tile and add their accumulators through LDS (K % 256 == 0; tiles alone on a CU)
