@@ -83,9 +83,9 @@ def lds_bytes(c: dict) -> int:
     if c["KIND"] == "decode":
         return c["NS"] * c["BN"] * 128
     if c["KIND"] == "wavek" and c.get("SHARED"):     # one ring for the workgroup, or the padded fp32 C tile
-        return max(c["NS"] * (c["BM"] + c["BN"]) * 128, c["BM"] * (c["BN"] + 4) * 4)
-    if c["KIND"] == "wavek":     # per wave: the ring, or the padded fp32 partial tile if that is larger
-        return 4 * max(c["NS"] * (c["BM"] + c["BN"]) * 128, c["BM"] * (c["BN"] + 4) * 4)
+        return max(c["NS"] * (c["BM"] + c["BN"]) * 128, c["BM"] * (c["BN"] + 4) * 4 + (c["BM"] + c["BN"]) * 4)
+    if c["KIND"] == "wavek":     # per wave: the ring, or the padded fp32 partial tile (and the last k of an odd K) if that is larger
+        return 4 * max(c["NS"] * (c["BM"] + c["BN"]) * 128, c["BM"] * (c["BN"] + 4) * 4 + (c["BM"] + c["BN"]) * 4)
     return c.get("KG", 1) * 2 * (c["BM"] + c["BN"]) * 128
 
 
@@ -117,13 +117,13 @@ def is_valid_config(c: dict) -> bool:
         # 2 x 2 waves over the tile, one ring: per wave and stage (BM + BN) / 32 loads, NS - 1 stages outstanding
         return (c["BM"] % 32 == 0 and c["BN"] % 32 == 0 and c["NS"] >= 3
                 and (c["NS"] - 1) * ((c["BM"] + c["BN"]) // 32) <= 63
-                and c["BM"] * c["BN"] // 4 % 256 == 0
+                and c["BM"] * c["BN"] // 4 % 256 == 0 and c["BM"] + c["BN"] <= 256
                 and lds_bytes(c) * c.get("OCC", 1) <= 160 * 1024)
     if c["KIND"] == "wavek":
         # per wave and ring stage (BM + BN) / 8 direct-to-LDS loads, NS stages outstanding
         return (c["BM"] % 16 == 0 and c["BN"] % 16 == 0 and c["NS"] >= 1
                 and (c["NS"] - 1) * ((c["BM"] + c["BN"]) // 8) <= 63
-                and c["BM"] * c["BN"] // 4 % 256 == 0
+                and c["BM"] * c["BN"] // 4 % 256 == 0 and c["BM"] + c["BN"] <= 256
                 and (c["BM"] // 16) * (c["BN"] // 16) * 4 <= 256
                 and lds_bytes(c) * c.get("OCC", 1) <= 160 * 1024)
     kg = c.get("KG", 1)
