@@ -103,6 +103,7 @@ def _check_unit(src: Path, obj: Path) -> None:
     isa_check.check_m0(src.name, text, need_kernels=8 if cfg["KIND"] == "mfma16" else 1)
     if cfg["KIND"] == "mfma16" and cfg.get("EFF"):
         isa_check.check_no_scratch(src.name, text)
+    isa_check.check_lds_bytes(src.name, text, kc.lds_bytes(cfg))
 
 
 def _compile(src: Path, force: bool) -> Path:

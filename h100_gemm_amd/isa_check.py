@@ -74,3 +74,15 @@ def check_no_scratch(unit: str, text: str) -> int:
         if sz != 0:
             raise IsaCheckError(f"{unit}: {n} uses {sz} bytes of scratch per lane")
     return len(aligned)
+
+
+def check_lds_bytes(unit: str, text: str, expected: int) -> int:
+    """The largest LDS allocation among a unit's kernels is what the config table says (the
+    table's figure decides how many workgroups the time model lets share a CU and is what
+    `mi_gemm_config_lds_bytes` reports).  Returns how many kernel descriptors were read."""
+    sizes = [int(v) for v in re.findall(r"\.amdhsa_group_segment_fixed_size (\d+)", text)]
+    if not sizes:
+        raise IsaCheckError(f"{unit}: no kernel descriptor with an LDS size found")
+    if max(sizes) != expected:
+        raise IsaCheckError(f"{unit}: kernels allocate up to {max(sizes)} bytes of LDS, the config table says {expected}")
+    return len(sizes)

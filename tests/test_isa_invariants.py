@@ -41,6 +41,17 @@ def test_aligned_kernels_do_not_spill():
         assert isa_check.check_no_scratch(name, text) >= 2
 
 
+def test_lds_sizes_match_the_config_table():
+    """What the compiled kernels allocate is what `kernel_configs.lds_bytes` says (the rules
+    for workgroups per CU and the C ABI's config query are derived from it)."""
+    units = built_units(("tile", "ring", "ring16", "mfma16", "decode", "stream", "wavek"))
+    assert len(units) == len(kc.CONFIGS)
+    for name, c, text in units:
+        assert isa_check.check_lds_bytes(name, text, kc.lds_bytes(c)) >= 1
+    with pytest.raises(isa_check.IsaCheckError, match="bytes of LDS"):
+        isa_check.check_lds_bytes(units[0][0], units[0][2], kc.lds_bytes(units[0][1]) - 1024)
+
+
 KERNEL = """_ZN2mi4testE:
 	s_load_dwordx2 s[0:1], s[4:5], 0x0
 {body}
