@@ -113,7 +113,13 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int M = p.M, N = p.N, K = p.K;
+    // split-K (gridDim.y pieces, the host's choice for few tiles with a very long K): this
+    // workgroup takes k_per_split of K from k0 on (a multiple of 64: rows keep their alignment)
+    // and leaves its sums in the workspace as fp32; splitk_reduce_kernel adds the pieces
+    const int k0 = p.splits > 1 ? (int)blockIdx.y * p.k_per_split : 0;
+    const int M = p.M, N = p.N, K = p.splits > 1 && p.K - k0 > p.k_per_split ? p.k_per_split : p.K - k0;
+    const unsigned char* A0 = (const unsigned char*)p.A + (size_t)k0 * 2;
+    const unsigned char* B0 = (const unsigned char*)p.B + (size_t)k0 * 2;
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     int tm, tn;
     tile_of_block<4>(blockIdx.x, gridDim.x, tiles_m, tiles_n, tm, tn);
@@ -125,21 +131,12 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
     const int KT = (Ke + 63) / 64;                           // units of K; the last may be partial
     const int tail_chunks = ((Ke & 63) + 7) >> 3;            // 16-byte chunks of a row in a partial last unit (0: none)
     const int tail_elems = Ke & 7;                           // elements of k < Ke in the last of them (0: all eight)
-    // the last k of an odd K: one element per row of the A and B panels, asked for now, put into
-    // LDS after the loops (rows outside M or N count as zero)
-    float last_elem = 0.0f;
-    if ((K & 1) != 0 && tid < BM + BN) {
-        const bool of_a = tid < BM;
-        const int r = of_a ? row0 + tid : col0 + tid - BM;
-        if (r < (of_a ? M : N))
-            last_elem = load_elem<DT>(of_a ? p.A : p.B, (size_t)r * (of_a ? p.lda : p.ldb) + K - 1);
-    }
     const int cnt = (KT - wave + 3) / 4;                     // units of this wave: wave, wave+4, ...
 
     const int rowsA = (M - row0) < BM ? (M - row0) : BM;
     const int rowsB = (N - col0) < BN ? (N - col0) : BN;
-    const unsigned char* Ab = (const unsigned char*)p.A + (size_t)row0 * p.lda * 2;
-    const unsigned char* Bb = (const unsigned char*)p.B + (size_t)col0 * p.ldb * 2;
+    const unsigned char* Ab = A0 + (size_t)row0 * p.lda * 2;
+    const unsigned char* Bb = B0 + (size_t)col0 * p.ldb * 2;
     const uint32_t bytesA = (uint32_t)((rowsA - 1) * p.lda + K) * 2u;
     const uint32_t bytesB = (uint32_t)((rowsB - 1) * p.ldb + K) * 2u;
     const __amdgpu_buffer_rsrc_t rsrcA = __builtin_amdgcn_make_buffer_rsrc((void*)Ab, 0, (int)bytesA, 0x00020000);
@@ -250,7 +247,18 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
     // entry t of the last-k row (fetched by thread t) sits behind the tile of wave t / 64, which
     // that wave is done with; the other waves may still be in their loops
     auto last_k = [&](int t) { return (float*)(lds + (t >> 6) * REGION + Cfg::TILE) + (t & 63); };
-    if (tid < BM + BN) *last_k(tid) = last_elem;
+    // the last k of an odd K: one element per row of the A and B panels into LDS (rows outside
+    // M or N count as zero).  Fetched here, not ahead of the loops: a register held across them
+    // and a store for every K cost the even K 1-4 % (the shared ring most), this costs the odd
+    // K nothing measurable
+    if ((K & 1) != 0 && tid < BM + BN) {
+        const bool of_a = tid < BM;
+        const int r = of_a ? row0 + tid : col0 + tid - BM;
+        float last_elem = 0.0f;
+        if (r < (of_a ? M : N))
+            last_elem = load_elem<DT>(of_a ? A0 : B0, (size_t)r * (of_a ? p.lda : p.ldb) + K - 1);
+        *last_k(tid) = last_elem;
+    }
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
@@ -259,6 +267,13 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
     __syncthreads();
     const bool scaled = p.alpha != 1.0f || p.beta != 0.0f;
     const bool c_vec_ok = (N & 3) == 0 && (p.ldc & 3) == 0 && ((uintptr_t)p.C & 7u) == 0;
+    // The usual calls -- alpha 1, beta 0 and an even K in one piece with rows of C in whole
+    // 8-byte groups (1) or not (3), an odd K in one piece (4), a piece of an even K (2) -- each
+    // take a copy of the loop without the branches of the others: with them in the loop every
+    // group of four waits for its LDS reads on its own (96x96 tiles: 0.5 us per launch).
+    auto store_c = [&](auto mode_c) __attribute__((always_inline)) {
+    constexpr int MODE = decltype(mode_c)::value;
+    constexpr bool PLAIN = MODE == 1, PIECE = MODE == 2, BY_ELEMENT = MODE == 3, ODD = MODE == 4, ANY = MODE == 0;
 #pragma unroll
     for (int it = 0; it < Cfg::QUADS; ++it) {
         const int q = it * 256 + tid;
@@ -269,13 +284,18 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
             const f32x4_t v = *(const f32x4_t*)((const float*)(lds + w * REGION) + m * PITCH + n);
             sum[0] += v[0]; sum[1] += v[1]; sum[2] += v[2]; sum[3] += v[3];
         }
-        if ((K & 1) != 0) {                                  // the last k of an odd K
+        if (ODD || (ANY && (K & 1) != 0)) {                  // the last k of an odd K
             const float a_last = *last_k(m);
             const f32x4_t b_last = *(const f32x4_t*)last_k(BM + n);
 #pragma unroll
             for (int e = 0; e < 4; ++e) sum[e] += a_last * b_last[e];
         }
-        if (scaled) {
+        if (PIECE || (ANY && p.splits > 1)) {                // (N % 4 == 0 is a launch precondition of split-K)
+            if (row0 + m < M && col0 + n < N)
+                *(f32x4_t*)(p.ws + ((size_t)blockIdx.y * M + row0 + m) * N + col0 + n) = sum;
+            continue;
+        }
+        if (ANY && scaled) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) sum[e] = mul_add_unfused(sum[e], p.alpha, p.beta);
         }
@@ -284,7 +304,7 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
             w2[0] = cvt_store2<DT>(sum[0], sum[1]);
             w2[1] = cvt_store2<DT>(sum[2], sum[3]);
             unsigned char* dst = (unsigned char*)p.C + ((size_t)(row0 + m) * p.ldc + col0 + n) * 2;
-            if (c_vec_ok) {                                  // every group of four starts on an 8-byte boundary inside N
+            if (PLAIN || (!BY_ELEMENT && c_vec_ok)) {        // every group of four starts on an 8-byte boundary inside N
                 *(u32x2_t*)dst = w2;
             } else {                                         // any N, any 2-byte aligned C: element by element
 #pragma unroll
@@ -293,6 +313,12 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
             }
         }
     }
+    };
+    if ((K & 1) == 0 && p.splits > 1) store_c(std::integral_constant<int, 2>{});
+    else if (p.splits > 1 || scaled) store_c(std::integral_constant<int, 0>{});
+    else if ((K & 1) != 0) store_c(std::integral_constant<int, 4>{});
+    else if (c_vec_ok) store_c(std::integral_constant<int, 1>{});
+    else store_c(std::integral_constant<int, 3>{});
 }
 
 // ---------------------------------------------------------------------------------------
@@ -342,7 +368,13 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
-    const int M = p.M, N = p.N, K = p.K;
+    // split-K (gridDim.y pieces, the host's choice for few tiles with a very long K): this
+    // workgroup takes k_per_split of K from k0 on (a multiple of 64: rows keep their alignment)
+    // and leaves its sums in the workspace as fp32; splitk_reduce_kernel adds the pieces
+    const int k0 = p.splits > 1 ? (int)blockIdx.y * p.k_per_split : 0;
+    const int M = p.M, N = p.N, K = p.splits > 1 && p.K - k0 > p.k_per_split ? p.k_per_split : p.K - k0;
+    const unsigned char* A0 = (const unsigned char*)p.A + (size_t)k0 * 2;
+    const unsigned char* B0 = (const unsigned char*)p.B + (size_t)k0 * 2;
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     int tm, tn;
     tile_of_block<4>(blockIdx.x, gridDim.x, tiles_m, tiles_n, tm, tn);
@@ -354,20 +386,11 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
     const int KT = (Ke + 63) / 64;                           // units of K; the last may be partial
     const int tail_chunks = ((Ke & 63) + 7) >> 3;            // 16-byte chunks of a row in a partial last unit (0: none)
     const int tail_elems = Ke & 7;                           // elements of k < Ke in the last of them (0: all eight)
-    // the last k of an odd K: one element per row of the A and B panels, asked for now, put into
-    // LDS after the loops (rows outside M or N count as zero)
-    float last_elem = 0.0f;
-    if ((K & 1) != 0 && tid < BM + BN) {
-        const bool of_a = tid < BM;
-        const int r = of_a ? row0 + tid : col0 + tid - BM;
-        if (r < (of_a ? M : N))
-            last_elem = load_elem<DT>(of_a ? p.A : p.B, (size_t)r * (of_a ? p.lda : p.ldb) + K - 1);
-    }
 
     const int rowsA = (M - row0) < BM ? (M - row0) : BM;
     const int rowsB = (N - col0) < BN ? (N - col0) : BN;
-    const unsigned char* Ab = (const unsigned char*)p.A + (size_t)row0 * p.lda * 2;
-    const unsigned char* Bb = (const unsigned char*)p.B + (size_t)col0 * p.ldb * 2;
+    const unsigned char* Ab = A0 + (size_t)row0 * p.lda * 2;
+    const unsigned char* Bb = B0 + (size_t)col0 * p.ldb * 2;
     const uint32_t bytesA = (uint32_t)((rowsA - 1) * p.lda + K) * 2u;
     const uint32_t bytesB = (uint32_t)((rowsB - 1) * p.ldb + K) * 2u;
     const __amdgpu_buffer_rsrc_t rsrcA = __builtin_amdgcn_make_buffer_rsrc((void*)Ab, 0, (int)bytesA, 0x00020000);
@@ -524,7 +547,18 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
     // acc[i][j][e] of lane l is C[m][n], m = wm*TM + i*16 + (l & 15), n = wn*TN + j*16 + 4*(l >> 4) + e
     float* part = (float*)lds;
     float* last_k = (float*)(lds + Cfg::TILE);
-    if (tid < BM + BN) last_k[tid] = last_elem;
+    // the last k of an odd K: one element per row of the A and B panels into LDS (rows outside
+    // M or N count as zero).  Fetched here, not ahead of the loops: a register held across them
+    // and a store for every K cost the even K 1-4 % (the shared ring most), this costs the odd
+    // K nothing measurable
+    if ((K & 1) != 0 && tid < BM + BN) {
+        const bool of_a = tid < BM;
+        const int r = of_a ? row0 + tid : col0 + tid - BM;
+        float last_elem = 0.0f;
+        if (r < (of_a ? M : N))
+            last_elem = load_elem<DT>(of_a ? A0 : B0, (size_t)r * (of_a ? p.lda : p.ldb) + K - 1);
+        last_k[tid] = last_elem;
+    }
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
@@ -533,18 +567,30 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
     __syncthreads();
     const bool scaled = p.alpha != 1.0f || p.beta != 0.0f;
     const bool c_vec_ok = (N & 3) == 0 && (p.ldc & 3) == 0 && ((uintptr_t)p.C & 7u) == 0;
+    // The usual calls -- alpha 1, beta 0 and an even K in one piece with rows of C in whole
+    // 8-byte groups (1) or not (3), an odd K in one piece (4), a piece of an even K (2) -- each
+    // take a copy of the loop without the branches of the others: with them in the loop every
+    // group of four waits for its LDS reads on its own (96x96 tiles: 0.5 us per launch).
+    auto store_c = [&](auto mode_c) __attribute__((always_inline)) {
+    constexpr int MODE = decltype(mode_c)::value;
+    constexpr bool PLAIN = MODE == 1, PIECE = MODE == 2, BY_ELEMENT = MODE == 3, ODD = MODE == 4, ANY = MODE == 0;
 #pragma unroll
     for (int it = 0; it < Cfg::QUADS; ++it) {
         const int q = it * 256 + tid;
         const int m = q / (BN / 4), n = (q % (BN / 4)) * 4;
         f32x4_t sum = *(const f32x4_t*)(part + m * PITCH + n);
-        if ((K & 1) != 0) {                                  // the last k of an odd K
+        if (ODD || (ANY && (K & 1) != 0)) {                  // the last k of an odd K
             const float a_last = last_k[m];
             const f32x4_t b_last = *(const f32x4_t*)(last_k + BM + n);
 #pragma unroll
             for (int e = 0; e < 4; ++e) sum[e] += a_last * b_last[e];
         }
-        if (scaled) {
+        if (PIECE || (ANY && p.splits > 1)) {                // (N % 4 == 0 is a launch precondition of split-K)
+            if (row0 + m < M && col0 + n < N)
+                *(f32x4_t*)(p.ws + ((size_t)blockIdx.y * M + row0 + m) * N + col0 + n) = sum;
+            continue;
+        }
+        if (ANY && scaled) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) sum[e] = mul_add_unfused(sum[e], p.alpha, p.beta);
         }
@@ -553,7 +599,7 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
             w2[0] = cvt_store2<DT>(sum[0], sum[1]);
             w2[1] = cvt_store2<DT>(sum[2], sum[3]);
             unsigned char* dst = (unsigned char*)p.C + ((size_t)(row0 + m) * p.ldc + col0 + n) * 2;
-            if (c_vec_ok) {                                  // every group of four starts on an 8-byte boundary inside N
+            if (PLAIN || (!BY_ELEMENT && c_vec_ok)) {        // every group of four starts on an 8-byte boundary inside N
                 *(u32x2_t*)dst = w2;
             } else {                                         // any N, any 2-byte aligned C: element by element
 #pragma unroll
@@ -562,18 +608,34 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
             }
         }
     }
+    };
+    if ((K & 1) == 0 && p.splits > 1) store_c(std::integral_constant<int, 2>{});
+    else if (p.splits > 1 || scaled) store_c(std::integral_constant<int, 0>{});
+    else if ((K & 1) != 0) store_c(std::integral_constant<int, 4>{});
+    else if (c_vec_ok) store_c(std::integral_constant<int, 1>{});
+    else store_c(std::integral_constant<int, 3>{});
+}
+
+// the second launch of a split-K run: the pieces' sums added in order, scaled, rounded once
+template <int DT>
+hipError_t launch_splitk_reduce(const DecodeArgs& a, hipStream_t stream) {
+    const size_t quads = ((size_t)a.M * a.N + 3) / 4;
+    return launch_kernel(splitk_reduce_kernel<DT>, dim3((unsigned)((quads + 255) / 256)), dim3(256), stream,
+                         a.ws, a.C, a.M, a.N, a.ldc, a.splits, a.alpha, a.beta);
 }
 
 template <class Cfg>
 hipError_t launch_shared_ring_kernel(const DecodeArgs& a, hipStream_t stream) {
     const int tiles = ((a.M + Cfg::BM - 1) / Cfg::BM) * ((a.N + Cfg::BN - 1) / Cfg::BN);
-    return launch_kernel(gemm_shared_ring_kernel<Cfg>, dim3(tiles), dim3(256), stream, a);
+    hipError_t e = launch_kernel(gemm_shared_ring_kernel<Cfg>, dim3(tiles, a.splits), dim3(256), stream, a);
+    return e != hipSuccess || a.splits == 1 ? e : launch_splitk_reduce<Cfg::DT>(a, stream);
 }
 
 template <class Cfg>
 hipError_t launch_wavek_kernel(const DecodeArgs& a, hipStream_t stream) {
     const int tiles = ((a.M + Cfg::BM - 1) / Cfg::BM) * ((a.N + Cfg::BN - 1) / Cfg::BN);
-    return launch_kernel(gemm_wavek_kernel<Cfg>, dim3(tiles), dim3(256), stream, a);
+    hipError_t e = launch_kernel(gemm_wavek_kernel<Cfg>, dim3(tiles, a.splits), dim3(256), stream, a);
+    return e != hipSuccess || a.splits == 1 ? e : launch_splitk_reduce<Cfg::DT>(a, stream);
 }
 
 }  // namespace mi

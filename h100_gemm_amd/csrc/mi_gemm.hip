@@ -108,6 +108,27 @@ int choose_tile_splits(const mi::KernelEntry& e, int M, int N, int K, bool split
     return mi::best_splits(e, M, N, K, true, ptr_aligned, cus, k_per_split, nullptr);
 }
 
+// Split-K for the small-tile kernels: an output of a few tiles with a very long K (128 x 384 x
+// 13376: 48 tiles of 32x32) leaves most CUs idle however small the tile, so K is cut into pieces
+// of whole 64-deep units, one workgroup per (tile, piece), as above.  The piece count comes from
+// the kernels' time model (best_wavek_splits).  MI_GEMM_SMALL_SPLITK=<n> forces a piece count
+// (1 = never split; tuning aid).
+int choose_small_tile_splits(const mi::KernelEntry& e, int M, int N, int K, bool splittable, int cus, int* k_per_split) {
+    *k_per_split = K;
+    static const int env = [] { const char* s = getenv("MI_GEMM_SMALL_SPLITK"); return s ? atoi(s) : 0; }();
+    if (!splittable || e.kind != mi::KIND_WAVEK || env == 1) return 1;
+    if (env > 1) {
+        int s = env < K / 128 ? env : K / 128;
+        if (s < 2 || (long long)s * M * N * 4 >= 0x7fffffffLL) return 1;
+        const int kps = ((K + s - 1) / s + 63) / 64 * 64;
+        s = (K + kps - 1) / kps;
+        if (s < 2) return 1;
+        *k_per_split = kps;
+        return s;
+    }
+    return mi::best_wavek_splits(e, M, N, K, true, cus, k_per_split, nullptr);
+}
+
 // ---- where the split-K kernels put their fp32 partial sums ----------------------------
 // Three sources, chosen by the entry point:
 //  * LIBRARY (mi_gemm_bf16 / _ex / _epilogue): one buffer per (device, stream), allocated on
@@ -336,6 +357,8 @@ Choice compute_choice(int requested, int M, int N, int K, bool streamable, bool 
         const int tiles_n = (N + e.BN - 1) / e.BN;
         c.splits = choose_splits(tiles_n, K, cus);   // no empty split
         c.k_per_split = ((K / 64 + c.splits - 1) / c.splits) * 64;
+    } else if (e.kind == mi::KIND_WAVEK) {
+        c.splits = choose_small_tile_splits(e, M, N, K, splittable, cus, &c.k_per_split);
     }
     return c;
 }
@@ -430,6 +453,16 @@ int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const vo
     if (e.kind == mi::KIND_WAVEK) {
         if (!shape_has_word_rows(K, A, B))
             return fail(MI_ERR_UNSUPPORTED, "config %s needs 4-byte aligned A and B", e.name);
+        args.splits = choice.splits;
+        args.k_per_split = choice.k_per_split;
+        if (args.splits > 1) {
+            const int wrc = acquire_workspace(wsrc, (size_t)args.splits * M * N * sizeof(float), (hipStream_t)stream, &args.ws);
+            if (wrc < 0) return wrc;
+            if (wrc > 0) {           // no workspace to be had: every tile walks all of K
+                args.splits = 1;
+                args.k_per_split = K;
+            }
+        }
         hipError_t err = e.launch[dtype][0](args, (hipStream_t)stream);
         if (err != hipSuccess)
             return fail(MI_ERR_HIP, "launch of %s failed: %s", e.name, hipGetErrorString(err));
@@ -539,7 +572,10 @@ int mi_gemm_config_grid(int config, int M, int N, int K) {
         return tiles_n * choose_splits(tiles_n, K, compute_units());
     }
     const int tiles = ((M + e.BM - 1) / e.BM) * ((N + e.BN - 1) / e.BN);
-    if (e.kind == mi::KIND_WAVEK) return tiles;
+    if (e.kind == mi::KIND_WAVEK) {    // split-K pieces, assuming an aligned C and no trace buffer
+        int kps = K;
+        return tiles * choose_small_tile_splits(e, M, N, K, N % 4 == 0, compute_units(), &kps);
+    }
     if (e.kind == mi::KIND_MFMA16) {   // split-K pieces, assuming an aligned C and no trace buffer
         int kps = K;
         return tiles * choose_tile_splits(e, M, N, K, N % 4 == 0, true, compute_units(), &kps);

@@ -233,6 +233,17 @@ def test_wave_split_k_kernels(mi, orc, config):
     check(mi, orc, 999, 1001, 1003, "uniform", config=config)
     check(mi, orc, 300, 201, 501, "normal", config=config, dtype=orc.FP16)
     check_epilogue(mi, orc, 300, 261, 1003, "int", -0.5, 2.75, config=config, exact=True)
+    # few tiles with a very long K: K cut into pieces over workgroups, fp32 sums of the pieces
+    # in the workspace, a second launch adds them -- whole units, a partial last unit, an odd
+    # K (all in the last piece), a last piece of a single unit; N % 4 != 0 does not split
+    assert mi.config_grid(config, 128, 384, 13376) > -(-128 // bm) * -(-384 // bn)
+    for M, N, K in [(128, 384, 13376), (bm, bn, 4096), (100, 36, 8200), (33, 8, 16390), (200, 132, 9001),
+                    (150, 100, 6002), (97, 101, 8193), (64, 64, 2112), (2 * bm + 1, bn + 4, 12352)]:
+        check(mi, orc, M, N, K, "int", config=config, exact=True)
+    check(mi, orc, 256, 256, 16384, "uniform", config=config)
+    check(mi, orc, 96, 200, 10001, "normal", config=config, dtype=orc.FP16)
+    check_epilogue(mi, orc, 200, 132, 9001, "int", -0.5, 2.75, config=config, exact=True)
+    check_epilogue(mi, orc, 132, 200, 8200, "int", 2.0, -1.0, config=config, c_layout=mi.MI_C_COL_MAJOR, exact=True)
     # operands that do not start on 4-byte boundaries are refused, not mis-computed
     for offA, offB in [(2, 0), (0, 6)]:
         with pytest.raises(mi.MiGemmError) as ei:

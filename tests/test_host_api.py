@@ -151,7 +151,12 @@ def test_config_table(mi):
             assert L.mi_gemm_config_supports(i, 0, 1000, 780, 4096) == 1
             assert L.mi_gemm_config_supports(i, 0, 1000, 777, 4098) == 1
             assert L.mi_gemm_config_supports(i, 0, 1, 1, 1) == 1
-            assert mi.config_grid(i, 1000, 780, 4097) == mi.config_grid(i, 1000, 780, 64)
+            # a long K may be cut into pieces (one workgroup per tile and piece) where N % 4 == 0
+            tiles = mi.config_grid(i, 1000, 780, 64)
+            grid = mi.config_grid(i, 1000, 780, 4097)
+            assert grid % tiles == 0 and 1 <= grid // tiles <= 4
+            assert mi.config_grid(i, 1000, 777, 4097) == -(-1000 // c["BM"]) * -(-777 // c["BN"])
+            assert mi.config_grid(i, 128, 384, 13376) > -(-128 // c["BM"]) * -(-384 // c["BN"])
         elif c.get("KG", 1) > 1:
             # K split over groups of waves inside the workgroup: any M, N; K in equal halves of whole double steps
             assert L.mi_gemm_config_supports(i, 0, 4095, 6143, 3072) == 1
