@@ -72,8 +72,8 @@ int mi_gemm_epilogue(int config, int dtype, int M, int N, int K, const void* A, 
                      void* C, float alpha, float beta, int c_layout, void* stream);
 
 /* ---- split-K workspace -----------------------------------------------------------------
- * Shapes with few output tiles and a long K (decode shapes with 32 < M <= 128, 512 x 512 x
- * 4096, ...) run as split-K: fp32 partial sums [pieces][M][N] go to a workspace and a second
+ * Shapes with few output tiles and a long K (decode shapes with 32 < M <= 128, 128 x 384 x
+ * 13376, 800 x 800 x 6000, ...) run as split-K: fp32 partial sums [pieces][M][N] go to a workspace and a second
  * kernel adds them in a fixed order.  The three entry points above take that workspace from
  * the library: one buffer per (device, stream), allocated on the first call that needs it,
  * replaced by a larger one on demand and never freed (an enqueued launch or a captured graph
