@@ -222,7 +222,9 @@ def _k(BM, BN, NS, WK=None, OCC=1, SHARED=0, WK_RAGGED=None, WK_ODD=None):
     if WK_ODD is not None:
         c["WK_ODD"] = WK_ODD           # a K unit's cost when K is odd, relative to an aligned pitch (default 2.0)
     if WK_RAGGED is not None:
-        c["WK_RAGGED"] = WK_RAGGED     # a K unit's cost when K % 64 != 0, relative to an aligned pitch (default 1.45)
+        # a K unit's cost when K % 64 != 0, relative to an aligned pitch: K % 8 == 0 with K < 2048 /
+        # K >= 2048, other even K with K < 2048 / K >= 2048 (default 1.15, 1.45, 1.45, 1.45)
+        c["WK_RAGGED"] = WK_RAGGED
     if SHARED:
         c["SHARED"] = 1         # 2 x 2 waves over the tile and one ring, instead of K split over the waves
     if OCC != 1:
@@ -271,16 +273,16 @@ CONFIGS = [
     _m(128, 128, 2, 2, DRAIN=1, KG=2, EFF=0.64, EFF_E=0.93),
     _d(128, NS=3),
     _d(64, NS=4),
-    _k(32, 32, NS=1, OCC=5, WK=(2.18, 0.0, 0.0775, 0.314), WK_ODD=1.95),
-    _k(32, 32, NS=2, OCC=2, WK=(1.71, 0.153, 0.0753, 0.580), WK_ODD=1.97),
-    _k(64, 32, NS=3, WK=(0.87, 2.10, 0.1188, 0.0), WK_ODD=2.05),
-    _k(64, 64, NS=1, OCC=2, WK=(1.93, 2.19, 0.1792, 0.0), WK_ODD=1.70),
-    _k(64, 64, NS=2, WK=(0.88, 2.81, 0.1648, 0.0), WK_ODD=1.97),
-    _k(96, 64, NS=2, WK=(1.35, 4.06, 0.2306, 0.0), WK_ODD=1.73),
-    _k(96, 96, NS=4, SHARED=1, WK=(1.03, 3.336, 0.3179, 0.0), WK_RAGGED=1.18, WK_ODD=1.58),
-    _k(64, 64, NS=4, SHARED=1, OCC=2, WK=(1.31, 1.734, 0.1815, 0.0), WK_ODD=1.77),
-    _k(96, 64, NS=4, SHARED=1, OCC=2, WK=(1.96, 1.90, 0.2313, 0.217), WK_ODD=1.72),
-    _k(64, 32, NS=4, SHARED=1, OCC=3, WK=(1.54, 1.362, 0.1234, 0.0), WK_ODD=1.92),
+    _k(32, 32, NS=1, OCC=5, WK=(2.18, 0.0, 0.0775, 0.314), WK_RAGGED=(1.26, 1.40, 1.46, 1.48), WK_ODD=1.95),
+    _k(32, 32, NS=2, OCC=2, WK=(1.71, 0.153, 0.0753, 0.580), WK_RAGGED=(1.19, 1.43, 1.55, 1.49), WK_ODD=1.97),
+    _k(64, 32, NS=3, WK=(0.87, 2.10, 0.1188, 0.0), WK_RAGGED=(1.21, 1.49, 1.83, 1.71), WK_ODD=2.05),
+    _k(64, 64, NS=1, OCC=2, WK=(1.93, 2.19, 0.1792, 0.0), WK_RAGGED=(1.00, 1.35, 1.34, 1.51), WK_ODD=1.70),
+    _k(64, 64, NS=2, WK=(0.88, 2.81, 0.1648, 0.0), WK_RAGGED=(1.11, 1.49, 1.67, 1.69), WK_ODD=1.97),
+    _k(96, 64, NS=2, WK=(1.35, 4.06, 0.2306, 0.0), WK_RAGGED=(0.85, 1.27, 1.25, 1.45), WK_ODD=1.73),
+    _k(96, 96, NS=4, SHARED=1, WK=(1.03, 3.336, 0.3179, 0.0), WK_RAGGED=(0.98, 1.24, 1.16, 1.37), WK_ODD=1.58),
+    _k(64, 64, NS=4, SHARED=1, OCC=2, WK=(1.31, 1.734, 0.1815, 0.0), WK_RAGGED=(1.06, 1.44, 1.31, 1.60), WK_ODD=1.77),
+    _k(96, 64, NS=4, SHARED=1, OCC=2, WK=(1.96, 1.90, 0.2313, 0.217), WK_RAGGED=(0.98, 1.32, 1.21, 1.52), WK_ODD=1.72),
+    _k(64, 32, NS=4, SHARED=1, OCC=3, WK=(1.54, 1.362, 0.1234, 0.0), WK_RAGGED=(1.20, 1.49, 1.49, 1.64), WK_ODD=1.92),
 ]
 
 assert all(is_valid_config(c) for c in CONFIGS), [config_name(c) for c in CONFIGS if not is_valid_config(c)]
