@@ -36,6 +36,9 @@ template takes (matmul_h100.cu.jinja:9-14) -- re-cast for CDNA4:
              tile): fixed + rounds of co-resident workgroups (tiles / (CUs x OCC), rounded up)
              x per round + tiles per CU (rounded up) x (per tile + K/64 x per unit);
              non-negative least squares on 89-99 shapes (the 96x64 shared-ring config: x 1.035); configs that carry it join the automatic choice
+    WK_RAGGED (wavek, optional) what a K unit costs more when K % 64 != 0 (rows that do not start on
+             128-byte lines): K % 8 == 0 with K < 2048 / K >= 2048, other even K with K < 2048 /
+             K >= 2048 (medians over 160 shapes of four lists); WK_ODD the same for an odd K
     EFF_E    (optional) throughput of the predicated variant relative to the aligned one, from
              7000^3, 6000^3 and 5000^3 (default 0.85); used for shapes the aligned variant cannot run
 
