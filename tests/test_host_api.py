@@ -218,6 +218,15 @@ def test_config_table(mi):
                     (8192, 8192, 28672), (0, 8, 8)]:
         assert mi.row_cut(M, N, K) == 0, (M, N, K)
     assert mi.workspace_bytes(7000, 7000, 7000) >= mi.workspace_bytes(88, 7000, 7000, config=mi.select_config(88, 7000, 7000))
+    # a few small tiles and a very long K: the small-tile kernels cut K over workgroups too, and
+    # the workspace query covers their pieces' sums; an odd N cannot be reduced and runs whole
+    c = mi.select_config(128, 384, 13376)
+    assert kc.CONFIGS[c]["KIND"] == "wavek"
+    pieces = mi.config_grid(c, 128, 384, 13376) // mi.config_grid(c, 128, 384, 64)
+    assert 2 <= pieces <= 16 and mi.workspace_bytes(128, 384, 13376) >= pieces * 128 * 384 * 4
+    assert mi.workspace_bytes(128, 383, 13376) == 0
+    assert kc.CONFIGS[mi.select_config(4828, 413, 13248)]["KIND"] == "wavek"    # narrow output, very long K: beyond 48 MB of operands
+    assert kc.CONFIGS[mi.select_config(448, 4864, 8192)]["KIND"] == "mfma16"
     # few tiles and a long K: split-K pieces of a tiled kernel fill the CUs
     c = mi.select_config(256, 8192, 8192)
     assert kc.CONFIGS[c]["KIND"] == "mfma16" and (kc.CONFIGS[c]["BM"], kc.CONFIGS[c]["BN"]) == (256, 128)
