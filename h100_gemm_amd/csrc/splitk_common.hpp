@@ -35,10 +35,12 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restr
     const size_t idx = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
     const size_t total = (size_t)M * N;
     if (idx >= total) return;
-    float4 a = *(const float4*)(ws + idx);
     // four pieces' loads in flight at a time, added in piece order (one load per trip made a
-    // reduction over 16 pieces a chain of 16 memory latencies)
-    int s = 1;
+    // reduction over 16 pieces a chain of 16 memory latencies); the sum starts from +0, which
+    // changes no bit of it (a piece's sums come out of accumulators that started from +0 and
+    // are never -0)
+    float4 a = {0.0f, 0.0f, 0.0f, 0.0f};
+    int s = 0;
     for (; s + 4 <= splits; s += 4) {
         const float4 b0 = *(const float4*)(ws + (size_t)s * total + idx);
         const float4 b1 = *(const float4*)(ws + (size_t)(s + 1) * total + idx);
@@ -49,7 +51,14 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restr
         a.x += b2.x; a.y += b2.y; a.z += b2.z; a.w += b2.w;
         a.x += b3.x; a.y += b3.y; a.z += b3.z; a.w += b3.w;
     }
-    for (; s < splits; ++s) {
+    if (s + 2 <= splits) {
+        const float4 b0 = *(const float4*)(ws + (size_t)s * total + idx);
+        const float4 b1 = *(const float4*)(ws + (size_t)(s + 1) * total + idx);
+        a.x += b0.x; a.y += b0.y; a.z += b0.z; a.w += b0.w;
+        a.x += b1.x; a.y += b1.y; a.z += b1.z; a.w += b1.w;
+        s += 2;
+    }
+    if (s < splits) {
         const float4 b = *(const float4*)(ws + (size_t)s * total + idx);
         a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
     }
