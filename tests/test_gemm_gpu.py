@@ -433,9 +433,10 @@ def test_random_shapes_small_tile_and_decode_kinds(mi, orc):
         if it % 2 == 1:
             # what only the small-tile kernels take: any K, any N, operands on 4-byte and C on
             # 2-byte boundaries
-            K = int(rng.choice([rng.integers(1, 80), rng.integers(80, 2600)]))
-            N = int(rng.integers(1, 720))
-            offA, offB, offC = 4 * int(rng.integers(0, 16)), 4 * int(rng.integers(0, 16)), 2 * int(rng.integers(0, 32))
+            # (a K beyond 2048 may be cut into pieces over workgroups where N % 4 == 0 and C is 8-byte aligned)
+            K = int(rng.choice([rng.integers(1, 80), rng.integers(80, 2600), rng.integers(2048, 9000)]))
+            N = int(rng.choice([rng.integers(1, 720), 4 * rng.integers(1, 180)]))
+            offA, offB, offC = 4 * int(rng.integers(0, 16)), 4 * int(rng.integers(0, 16)), int(rng.choice([2, 8])) * int(rng.integers(0, 8))
             pool = small
         able = [i for i in pool if mi._lib.load().mi_gemm_config_supports(i, 0, M, N, K)]
         config = -1 if it % 3 == 0 or not able else able[int(rng.integers(0, len(able)))]
