@@ -50,6 +50,8 @@ WORKLOADS = {
     "mid1440": (1440, 1440, 1472, "uniform"),
     "square1536": (1536, 1536, 1536, "uniform"),
     "square2048": (2048, 2048, 2048, "uniform"),
+    # 48 tiles of 32x32 with a very long K: K cut into pieces over workgroups in the small-tile kernel
+    "longk128": (128, 384, 13376, "uniform"),
 }
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (the summaries under
 # profiles/ give the commands), scaled by the same counters on a copy kernel of known size:
