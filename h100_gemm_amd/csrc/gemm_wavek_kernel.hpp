@@ -1,6 +1,6 @@
 // gemm_wavek_kernel.hpp -- gfx950 GEMM kernels for outputs of few tiles:
 //
-//   C[M,N] = A[M,K] . B[N,K]^T     small tiles, one kernel, no workspace
+//   C[M,N] = A[M,K] . B[N,K]^T     small tiles; one kernel and no workspace, except for a very long K
 //   gemm_wavek_kernel:        K split over the four waves of a workgroup (few tiles, long K)
 //   gemm_shared_ring_kernel:  2 x 2 waves over the tile, one shared ring (further down)
 //
@@ -49,6 +49,10 @@
 // groups of four elements do not all start on 8-byte boundaries inside N, C is stored element
 // by element.  Rows that start on 128-byte boundaries (K % 64 == 0, aligned bases) are what the
 // kernel is fastest on: with any other pitch every 128-byte piece of a row straddles two lines.
+// A very long K under an output of so few tiles that even these leave CUs idle (128 x 384 x 13376)
+// is cut into pieces of whole units, one workgroup per (tile, piece) on gridDim.y: the piece's
+// sums go to the workspace as fp32 and splitk_reduce_kernel adds the pieces (the host's choice,
+// DecodeArgs::splits; 19.9 -> 10.8 us there).
 // The reference has no counterpart: its kernels use one tile size (matmul_utils.cuh:362).
 #pragma once
 
