@@ -46,6 +46,9 @@ SYMBOLS = {
     "mi_gemm_epilogue_ws": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
                                       C.c_void_p, C.c_float, C.c_float, C.c_int, C.c_void_p, C.c_size_t,
                                       C.c_void_p]),
+    "mi_gemm_reserve_workspace": (C.c_int, [C.c_void_p, C.c_size_t]),
+    "mi_gemm_release_workspace": (C.c_int, [C.c_void_p]),
+    "mi_gemm_library_workspace_bytes": (C.c_size_t, []),
     "mi_gemm_bf16_noalloc": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "mi_reference_gpu_gemm": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
                                         C.c_void_p, C.c_float, C.c_float, C.c_void_p]),

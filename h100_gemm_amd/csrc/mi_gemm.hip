@@ -132,13 +132,15 @@ int choose_small_tile_splits(const mi::KernelEntry& e, int M, int N, int K, bool
 // ---- where the split-K kernels put their fp32 partial sums ----------------------------
 // Three sources, chosen by the entry point:
 //  * LIBRARY (mi_gemm_bf16 / _ex / _epilogue): one buffer per (device, stream), allocated on
-//    first use and replaced by a larger one on demand.  A buffer is never freed while the
-//    process lives: launches already enqueued and captured graphs keep its address, so a
-//    replaced buffer only moves to a retired list (sizes are powers of two, so the retired
-//    ones together stay below the live one).  Launches on one stream are ordered and
-//    launches on different streams use different buffers, so concurrent split-K calls do
-//    not meet.  A stream that is being captured cannot allocate: if it has no buffer that is
-//    large enough yet, the launch runs unsplit instead.
+//    first use and replaced by a larger one on demand.  Launches already enqueued and captured
+//    graphs keep a buffer's address, so a replaced buffer moves to the stream's retired list
+//    (sizes are powers of two, so the retired ones together stay below the live one) and
+//    nothing is freed behind the caller's back: mi_gemm_release_workspace frees a stream's
+//    buffers (after synchronising it), and the table holds at most kMaxStreamWs streams per
+//    device -- a further stream takes over an entry once the device is idle.  Launches on one
+//    stream are ordered and launches on different streams use different buffers, so
+//    concurrent split-K calls do not meet.  A stream that is being captured cannot allocate:
+//    if it has no buffer that is large enough yet, the launch runs unsplit instead.
 //  * CALLER (mi_gemm_epilogue_ws): the caller's buffer, nothing is allocated; too small (or
 //    NULL) means the launch runs unsplit.
 //  * STATIC (mi_gemm_bf16_noalloc): the file-scope device array below, one copy per GPU the
@@ -159,13 +161,18 @@ struct StreamWs {
     hipStream_t stream;
     float* ptr;
     size_t bytes;
+    std::vector<void*> retired;      // buffers this stream outgrew: an enqueued launch or a captured graph may still
+                                     // hold their address, so they live until the stream's workspace is released
 };
 struct DeviceState {
-    std::vector<StreamWs> ws;        // live buffers, one per stream that ran a split-K launch
-    std::vector<void*> retired;      // replaced buffers: kept until the process ends
+    std::vector<StreamWs> ws;        // one entry per stream that ran a split-K launch (at most kMaxStreamWs)
     unsigned char* scratch = nullptr;   // device address of `scratch` on this device
     int cus = 0;
 };
+// Streams with a buffer of their own per device.  A process that keeps creating streams does not
+// grow the table beyond this: the next new stream waits for the device to go idle and takes over
+// an entry (see acquire_workspace), so at most this many live buffers exist per device.
+constexpr size_t kMaxStreamWs = 16;
 std::mutex g_ws_mutex;
 DeviceState g_dev[kMaxDevices];
 
@@ -189,6 +196,14 @@ hipError_t static_scratch(unsigned char** out) {
     }
     *out = st.scratch;
     return hipSuccess;
+}
+
+void free_entry(StreamWs& w) {
+    if (w.ptr) (void)hipFree(w.ptr);
+    for (void* r : w.retired) (void)hipFree(r);
+    w.ptr = nullptr;
+    w.bytes = 0;
+    w.retired.clear();
 }
 
 // 0: *out holds `bytes` of workspace; 1: none to be had without allocating where that is not
@@ -229,16 +244,41 @@ int acquire_workspace(const WsSource& src, size_t bytes, hipStream_t stream, flo
     if (cap != hipStreamCaptureStatusNone) return 1;
     size_t want = (size_t)4 << 20;
     while (want < bytes) want <<= 1;
+    if (!mine && st.ws.size() >= kMaxStreamWs) {
+        // The table is full (a process that keeps making streams, or never releases): once the
+        // device is idle no launch holds any buffer, so the smallest entry changes hands -- its
+        // buffer as it is when large enough, else freed here and replaced below.
+        hipError_t e = hipDeviceSynchronize();
+        if (e != hipSuccess)
+            return fail(MI_ERR_HIP, "hipDeviceSynchronize before reusing a split-K workspace failed: %s", hipGetErrorString(e));
+        StreamWs* take = nullptr;
+        for (StreamWs& w : st.ws)       // the smallest entry that is already large enough ...
+            if (w.bytes >= bytes && (!take || w.bytes < take->bytes)) take = &w;
+        if (!take)
+            for (StreamWs& w : st.ws)   // ... else the smallest of all
+                if (!take || w.bytes < take->bytes) take = &w;
+        for (void* r : take->retired) (void)hipFree(r);
+        take->retired.clear();
+        take->stream = stream;
+        if (take->bytes >= bytes) {
+            *out = take->ptr;
+            return 0;
+        }
+        if (take->ptr) (void)hipFree(take->ptr);
+        take->ptr = nullptr;
+        take->bytes = 0;
+        mine = take;
+    }
     float* p = nullptr;
     hipError_t e = hipMalloc((void**)&p, want);
     if (e != hipSuccess)
         return fail(MI_ERR_HIP, "split-K workspace allocation of %zu bytes failed: %s", want, hipGetErrorString(e));
     if (mine) {
-        st.retired.push_back(mine->ptr);
+        if (mine->ptr) mine->retired.push_back(mine->ptr);
         mine->ptr = p;
         mine->bytes = want;
     } else {
-        st.ws.push_back({stream, p, want});
+        st.ws.push_back({stream, p, want, {}});
     }
     *out = p;
     return 0;
@@ -328,6 +368,7 @@ int tuned_config(int M, int N, int K, bool streamable, bool small_ok) {
         const mi::KernelEntry& e = mi::kKernels[t.config];
         if ((is_split_k_decode(e.kind) || e.kind == mi::KIND_STREAM) && (!streamable || M > e.BM)) continue;
         if (e.kind == mi::KIND_WAVEK && !small_ok) continue;
+        if (e.kg > 1 && K % (128 * e.kg) != 0) continue;      // (the rule mi_gemm_config_supports applies)
         return t.config;
     }
     return -1;
@@ -405,10 +446,29 @@ int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const vo
         const int m1 = rows_to_cut(M, N, K, streamable, shape_is_splittable(N, C, DB),
                                    aligned16(A) && aligned16(B) && aligned16(C), shape_has_word_rows(K, A, B));
         if (m1 > 0) {
+            // Both parts' workspace is settled before anything is launched: a part that could not
+            // get its partial sums' room (the static array too small, an allocation that fails)
+            // must not leave the other part's rows of C written and the call failed.
+            const void* A2 = (const unsigned char*)A + (size_t)m1 * K * 2;
+            void* C2 = (unsigned char*)C + (size_t)m1 * N * 2;
+            size_t need = 0;
+            for (int part = 0; part < 2; ++part) {
+                const int Mp = part ? M - m1 : m1;
+                const void* Ap = part ? A2 : A;
+                const void* Cp = part ? C2 : C;
+                const Choice c = choose(config, Mp, N, K, shape_is_streamable(Mp, N, K, Ap, B, Cp), shape_is_splittable(N, Cp, nullptr),
+                                        aligned16(Ap) && aligned16(B) && aligned16(Cp), shape_has_word_rows(K, Ap, B));
+                const size_t b = c.splits > 1 ? (size_t)c.splits * Mp * N * sizeof(float) : 0;
+                if (b > need) need = b;
+            }
+            if (need > 0) {
+                float* unused = nullptr;
+                const int wrc = acquire_workspace(wsrc, need, (hipStream_t)stream, &unused);
+                if (wrc < 0) return wrc;
+            }
             rc = run_gemm(config, dtype, m1, N, K, A, B, C, nullptr, alpha, beta, stream, wsrc, false);
             if (rc != MI_OK) return rc;
-            return run_gemm(config, dtype, M - m1, N, K, (const unsigned char*)A + (size_t)m1 * K * 2, B,
-                            (unsigned char*)C + (size_t)m1 * N * 2, nullptr, alpha, beta, stream, wsrc, false);
+            return run_gemm(config, dtype, M - m1, N, K, A2, B, C2, nullptr, alpha, beta, stream, wsrc, false);
         }
     }
     // with a trace buffer the automatic choice stays with the kernels that fill it (the tiled
@@ -695,6 +755,38 @@ int mi_gemm_bf16_noalloc(int M, int N, int K, const uint16_t* A, const uint16_t*
     WsSource src;
     src.mode = WS_STATIC;
     return run_gemm(MI_CONFIG_AUTO, MI_DTYPE_BF16, M, N, K, A, B, C, nullptr, 1.0f, 0.0f, stream, src);
+}
+
+int mi_gemm_reserve_workspace(void* stream, size_t bytes) {
+    if (bytes == 0) return MI_OK;
+    float* p = nullptr;
+    const int rc = acquire_workspace(WsSource{}, bytes, (hipStream_t)stream, &p);
+    if (rc > 0) return fail(MI_ERR_UNSUPPORTED, "the stream is being captured: no workspace can be allocated now");
+    return rc < 0 ? rc : MI_OK;
+}
+
+int mi_gemm_release_workspace(void* stream) {
+    // NULL: every stream's buffers on the current device, once the device is idle
+    if (stream == nullptr) MI_HIP(hipDeviceSynchronize());
+    else MI_HIP(hipStreamSynchronize((hipStream_t)stream));
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    DeviceState& st = device_state();
+    for (size_t i = 0; i < st.ws.size();) {
+        if (stream == nullptr || st.ws[i].stream == (hipStream_t)stream) {
+            free_entry(st.ws[i]);
+            st.ws.erase(st.ws.begin() + (long)i);
+        } else {
+            ++i;
+        }
+    }
+    return MI_OK;
+}
+
+size_t mi_gemm_library_workspace_bytes(void) {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    size_t total = 0;
+    for (const StreamWs& w : device_state().ws) total += w.bytes;
+    return total;
 }
 
 int mi_reference_gpu_gemm(int dtype, int M, int N, int K, const void* A, const void* B, void* C,

@@ -75,15 +75,44 @@ int mi_gemm_epilogue(int config, int dtype, int M, int N, int K, const void* A, 
  * Shapes with few output tiles and a long K (decode shapes with 32 < M <= 128, 128 x 384 x
  * 13376, 800 x 800 x 6000, ...) run as split-K: fp32 partial sums [pieces][M][N] go to a workspace and a second
  * kernel adds them in a fixed order.  The three entry points above take that workspace from
- * the library: one buffer per (device, stream), allocated on the first call that needs it,
- * replaced by a larger one on demand and never freed (an enqueued launch or a captured graph
- * may still hold its address); a stream under capture that has no large enough buffer yet
- * runs the launch unsplit.  The reference's launchers allocate nothing per call
- * (matmul_h100_optimal.cu:32-59); the two functions below give a caller the same property:
- * it owns the workspace, per stream or per graph, and the library allocates nothing. */
+ * the library: one buffer per (device, stream), a power of two of at least 4 MiB, allocated on
+ * the first call that needs it and replaced by a larger one on demand; a replaced buffer is
+ * kept (an enqueued launch or a captured graph may still hold its address) until
+ * mi_gemm_release_workspace gives the stream's buffers back.  At most 16 streams per device
+ * hold a buffer: a further stream waits for the device to go idle (hipDeviceSynchronize) and
+ * takes over the smallest entry, so a process that keeps creating streams does not keep
+ * growing.  A stream under capture that has no large enough buffer yet runs the launch unsplit;
+ * a first or a growing use calls hipMalloc, which must not happen while ANY thread captures
+ * in hipStreamCaptureModeGlobal: reserve beforehand (mi_gemm_reserve_workspace) or use
+ * mi_gemm_epilogue_ws / mi_gemm_bf16_noalloc there.  The reference's launchers allocate
+ * nothing per call (matmul_h100_optimal.cu:32-59); mi_gemm_epilogue_ws gives a caller the
+ * same property: it owns the workspace, per stream or per graph, and the library allocates
+ * nothing. */
+
+/* Makes sure the library holds at least `bytes` of workspace for `stream` on the current
+ * device (allocating or growing now, at a time the caller chooses, instead of inside a later
+ * GEMM call).  MI_ERR_UNSUPPORTED when the stream is being captured.  The reference's launcher
+ * holds no per-call device memory (matmul_h100_optimal.cu:32-59); no counterpart there. */
+int mi_gemm_reserve_workspace(void* stream, size_t bytes);
+
+/* Gives the library's workspace buffers of `stream` on the current device back (the live one
+ * and the ones it outgrew), after hipStreamSynchronize(stream); NULL: the buffers of every
+ * stream of the current device, after hipDeviceSynchronize.  Graphs captured from split-K
+ * launches through the library on that stream must not be replayed afterwards.  Call it
+ * before destroying a stream that ran GEMMs: the table is keyed on the stream handle, and a
+ * later stream that gets the same handle value would otherwise inherit the buffer.  The
+ * reference's launcher holds no per-call device memory (matmul_h100_optimal.cu:32-59). */
+int mi_gemm_release_workspace(void* stream);
+
+/* Bytes of workspace the library currently holds for the streams of the current device (live
+ * buffers; 0 after mi_gemm_release_workspace(NULL)). */
+size_t mi_gemm_library_workspace_bytes(void);
 
 /* Bytes of workspace the library's choice of kernel wants for this call (0 when the shape
- * does not run split-K): the largest need over the pointer alignments a launch can meet. */
+ * does not run split-K).  An upper bound: the largest need over the pointer alignments a
+ * launch can meet and over the two parts of a shape whose rows the automatic choice cuts
+ * (2248 x 8192 x 28672: 210.75 MiB for the uncut split of an unaligned call, 25 MiB for the
+ * aligned call, which is cut at 2048 rows). */
 size_t mi_gemm_workspace_bytes(int config, int dtype, int M, int N, int K, int c_layout);
 
 /* mi_gemm_epilogue with a caller-owned workspace: `ws` is a device pointer, 16-byte aligned,
@@ -105,7 +134,10 @@ int mi_gemm_epilogue_ws(int config, int dtype, int M, int N, int K, const void* 
  * shares that GPU's array: calls that run split-K and overlap on one GPU (two streams, or a
  * graph replay next to eager calls) race on it -- keep them on one stream.  Nothing in the
  * array needs clearing between calls: the kernels write every partial sum they later read.
- * Results are bit-identical to mi_gemm_bf16 for the same arguments. */
+ * A shape whose rows the automatic choice cuts in two is refused as a whole, before anything
+ * is launched, when either part's partial sums do not fit.  Results are bit-identical to
+ * mi_gemm_bf16 for the same arguments wherever mi_gemm_bf16 runs the same split (it runs
+ * unsplit, a different summation order, on a capturing stream without a buffer). */
 #define MI_GEMM_NOALLOC_SCRATCH_BYTES ((size_t)32 << 20)
 int mi_gemm_bf16_noalloc(int M, int N, int K, const uint16_t* A, const uint16_t* B, uint16_t* C,
                          void* stream);

@@ -547,6 +547,84 @@ def test_split_k_workspace_growth_keeps_enqueued_launches_valid(mi, orc):
     assert hip.hipStreamDestroy(stream) == 0
 
 
+def test_library_workspace_is_released_and_its_table_capped(mi, orc):
+    """A server that creates and destroys streams: 64 streams in turn run the split-K decode
+    shape 128 x 8192 x 8192 through the library's own workspace.  The first half give their
+    buffer back before the stream is destroyed (mi_gemm_release_workspace), the second half
+    never do: the library then holds buffers for at most 16 streams.  After a release of
+    everything the device's free memory is back to within one buffer of where it started, and
+    every result is bit-exact."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    L = mi._lib.load()
+    M, N, K = 128, 8192, 8192
+    need = mi.workspace_bytes(M, N, K)
+    assert need > 0
+    buf = 4 << 20
+    while buf < need:
+        buf <<= 1
+    A, B = make_inputs(orc, M, N, K, "int")
+    ref = orc.reference_cpu_gemm(A, B)
+    d = Dev(mi, A, B, M, N)
+    mi._lib.check(L.mi_gemm_release_workspace(None))           # whatever earlier tests left
+    assert L.mi_gemm_library_workspace_bytes() == 0
+
+    def free_bytes():
+        f, t = ctypes.c_size_t(), ctypes.c_size_t()
+        assert hip.hipMemGetInfo(ctypes.byref(f), ctypes.byref(t)) == 0
+        return f.value
+
+    start = free_bytes()
+
+    def run_on(stream, tag):
+        d.dC.fill_bytes(0xFF)
+        mi._lib.check(L.mi_gemm_ex(-1, 0, M, N, K, d.dA.ptr, d.dB.ptr, d.dC.ptr, None, stream))
+        mi._lib.check(L.mi_stream_sync(stream))
+        C = d.dC.to_numpy((M, N), np.uint16)
+        assert (C == ref).all(), f"{tag}: {int((C != ref).sum())} elements differ"
+
+    for i in range(64):
+        stream = ctypes.c_void_p()
+        assert hip.hipStreamCreate(ctypes.byref(stream)) == 0
+        run_on(stream, f"stream {i}")
+        held = L.mi_gemm_library_workspace_bytes()
+        if i < 32:
+            assert held == buf, (i, held, buf)
+            mi._lib.check(L.mi_gemm_release_workspace(stream))
+            assert L.mi_gemm_library_workspace_bytes() == 0
+        else:
+            # never released: a later stream may get the destroyed one's handle value and with it
+            # its buffer; either way no more than the table's 16 entries
+            assert buf <= held <= 16 * buf, (i, held, buf)
+        assert hip.hipStreamDestroy(stream) == 0
+    # 24 streams alive at once: the table stops at 16 buffers, the others take one over
+    alive = []
+    for i in range(24):
+        stream = ctypes.c_void_p()
+        assert hip.hipStreamCreate(ctypes.byref(stream)) == 0
+        alive.append(stream)
+        run_on(stream, f"live stream {i}")
+        assert L.mi_gemm_library_workspace_bytes() <= 16 * buf
+    assert L.mi_gemm_library_workspace_bytes() == 16 * buf
+    for i, stream in enumerate(alive):                         # and again, every stream taking turns
+        run_on(stream, f"live stream {i}, second round")
+    assert L.mi_gemm_library_workspace_bytes() == 16 * buf
+    for stream in alive:
+        assert hip.hipStreamDestroy(stream) == 0
+    mi._lib.check(L.mi_gemm_release_workspace(None))
+    assert L.mi_gemm_library_workspace_bytes() == 0
+    assert abs(free_bytes() - start) <= buf, (free_bytes(), start, buf)
+    # a reservation made ahead of the first GEMM is what that GEMM then uses
+    mi._lib.check(L.mi_gemm_reserve_workspace(None, need))
+    assert L.mi_gemm_library_workspace_bytes() == buf
+    d.dC.fill_bytes(0xFF)
+    mi._lib.check(L.mi_gemm_ex(-1, 0, M, N, K, d.dA.ptr, d.dB.ptr, d.dC.ptr, None, None))
+    mi.synchronize()
+    assert (d.dC.to_numpy((M, N), np.uint16) == ref).all()
+    assert L.mi_gemm_library_workspace_bytes() == buf
+    mi._lib.check(L.mi_gemm_release_workspace(None))
+
+
 def test_caller_workspace_launches_on_two_streams(mi, orc):
     """mi_gemm_epilogue_ws: split-K partial sums in buffers the caller owns, one per stream;
     interleaved launches on two streams, bit-exact on the integer fill and bit-identical to

@@ -64,3 +64,24 @@ def test_noalloc_entry_point_refuses_what_does_not_fit(mi, orc):
     assert b"static scratch array" in L.mi_last_error()
     assert L.mi_gemm_bf16_noalloc(0, N, K, dA.ptr, dB.ptr, dC.ptr, None) == mi._lib.MI_ERR_INVALID
     mi.synchronize()
+
+
+def test_noalloc_entry_point_refuses_a_cut_shape_before_it_writes_anything(mi, orc):
+    """A large ragged shape that the automatic choice runs as two GEMMs (the first 2048 rows,
+    then the rest) and whose second part would need more partial sums than the array holds:
+    the call is refused before the first part is launched, so C is untouched."""
+    L = mi._lib.load()
+    M, N, K = 2298, 8192, 32768
+    assert mi.row_cut(M, N, K) > 0
+    dA, dB, dC = mi.DeviceBuffer(M * K * 2), mi.DeviceBuffer(N * K * 2), mi.DeviceBuffer(M * N * 2)
+    dA.fill_bytes(0)
+    dB.fill_bytes(0)
+    dC.fill_bytes(0xFF)
+    rc = L.mi_gemm_bf16_noalloc(M, N, K, dA.ptr, dB.ptr, dC.ptr, None)
+    mi.synchronize()
+    assert rc == mi._lib.MI_ERR_UNSUPPORTED, rc
+    assert b"static scratch array" in L.mi_last_error()
+    C = dC.to_numpy((M, N), np.uint16)
+    assert (C == 0xFFFF).all(), f"{int((C != 0xFFFF).sum())} elements of C were written by a refused call"
+    for b in (dA, dB, dC):
+        b.free()
