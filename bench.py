@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """bench.py -- headline benchmark: bf16 GEMM TFLOP/s at M=N=K=8192 on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--config NAME]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--config NAME] [--no-configs]
 
 One "step" is one launch of the GEMM (A 8192x8192 row-major, B 8192x8192 K-major, both
 U[-1,1) seeded bf16, C bf16, fp32 accumulate) with the inputs already resident in HBM.
@@ -9,7 +9,10 @@ Prints ONE JSON line.  `value` = 2*M*N*K / time per launch, in TFLOP/s.  The `ro
 object prices the kernel against MI355X's published dense bf16 MFMA peak (2.5 PFLOP/s);
 for the HBM-bound skinny workloads it is priced against 8 TB/s instead.  `cpu_baseline` is
 the CPU restatement of the reference's reference_cpu_gemm (reference.h:5-46) timed on this
-box's host cores on a bounded sample of 64x64 output tiles of the same problem.
+box's host cores on a bounded sample of 64x64 output tiles of the same problem.  After the
+headline's timed region the other seven shapes of the benchmark definition (512^3, the two MLP
+shapes, the three decode shapes, 4095x6143x3073) are timed with the library's own kernel choice
+and reported as `configs`, one row each with its roofline fraction and tolerance check.
 
 The timed region is bracketed by device synchronisation and measured with HIP events
 recorded on the stream the kernel is launched on (the null stream, as the reference's
@@ -53,24 +56,41 @@ WORKLOADS = {
     # 48 tiles of 32x32 with a very long K: K cut into pieces over workgroups in the small-tile kernel
     "longk128": (128, 384, 13376, "uniform"),
 }
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (the summaries under
-# profiles/ give the commands), scaled by the same counters on a copy kernel of known size:
+# HBM-side bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (the summaries
+# under profiles/ give the commands), scaled by the same counters on a copy kernel of known size:
 # FETCH_SIZE counts KiB and reads half of what a plain 256 MiB device copy moves (131087 for
 # 262144 KiB read), so it is scaled by 2.0; WRITE_SIZE reads the copy's writes exactly (1.0).
-# workload -> (kernel configuration the counters were read on, bytes).  A profile constant,
-# not something this run measures: reported only while the run uses that same kernel.
-MEASURED_TRAFFIC_BYTES = {
-    "square8192": ("m256x256_w2x2_g4_b3", (787026 * 2.0 + 131083) * 1024),     # 1.75 GB against 0.40 GB algorithmic
-    "skinny16": ("s16x32_n5", (66589.6 * 2.0 + 256) * 1024),         # 0.137 GB: B is read exactly once
-    "unaligned": ("m256x192_w2x2_g4_b3", (130105 * 2.0 + 49737) * 1024),       # 0.317 GB against 0.113 GB algorithmic
-    "mlp_up": ("m256x256_w2x2_g4_b3", (2753408 * 2.0 + 458779) * 1024),         # 6.1 GB against 1.34 GB algorithmic
-    "mlp_down": ("m256x256_w2x2_g8_b1", (2.7535e6 * 2.0 + 131072) * 1024),      # 5.8 GB against 1.07 GB algorithmic
-    "square512": ("k32x32_n2", (1569.0 * 2.0 + 512) * 1024),           # 3.6 MB against 1.5 MB algorithmic: a copy of the rows per L2
-    "fewtile512": ("k32x32_n2", (12321.0 * 2.0 + 512) * 1024),         # 25.8 MB against 8.9 MB algorithmic
-    "fewtile1024": ("k64x64_n2", (24626.5 * 2.0 + 2048) * 1024),       # 52.5 MB against 18.9 MB algorithmic
-    "skinny64": ("d64x128_n4", ((69689 + 4114) * 2.0 + 8192 + 1024) * 1024),     # main + reduce kernels
-    "skinny128": ("d128x128_n3", ((73797 + 8210) * 2.0 + 16384 + 2048) * 1024),   # main + reduce kernels
+# workload -> (kernel configuration the counters were read on, profile that holds the figures,
+# FETCH_SIZE KiB of each kernel of the launch, WRITE_SIZE KiB of each).  Profile constants, not
+# something this run measures: reported only while the run uses that same kernel; the figures are
+# the ones the named profile shows (tests/test_host_api.py compares them).
+FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
+MEASURED_TRAFFIC_KIB = {
+    "square8192": ("m256x256_w2x2_g4_b3", "gemm_mfma16_kernel_square8192.md", (786705,), (131081,)),   # 1.75 GB against 0.40 GB algorithmic
+    "skinny16": ("s16x32_n5", "gemm_stream_kernel_skinny16.md", (66589,), (256,)),                     # 0.137 GB: B is read exactly once
+    "unaligned": ("m256x192_w2x2_g4_b3", "gemm_mfma16_kernel_unaligned.md", (130077,), (49670,)),      # 0.317 GB against 0.113 GB algorithmic
+    "mlp_up": ("m256x256_w2x2_g4_b3", "gemm_mfma16_kernel_mlp_up.md", (2753369,), (458767,)),          # 6.1 GB against 1.34 GB algorithmic
+    "mlp_down": ("m256x256_w2x2_g8_b1", "gemm_mfma16_kernel_mlp_down.md", (2752957,), (131159,)),      # 5.8 GB against 1.07 GB algorithmic
+    "square512": ("k32x32_n2", "gemm_wavek_kernel_square512.md", (1565,), (512,)),                     # 3.7 MB against 1.5 MB algorithmic: a copy of the rows per L2
+    "fewtile512": ("k32x32_n2", "gemm_wavek_kernel_fewtile.md", (12317,), (512,)),                     # 25.8 MB against 8.9 MB algorithmic
+    "fewtile1024": ("k64x64_n2", "gemm_wavek_kernel_fewtile.md", (24627,), (2048,)),                   # 52.5 MB against 18.9 MB algorithmic
+    "skinny64": ("d64x128_n4", "gemm_decode_kernel_skinny128_skinny64.md", (69689, 4114), (8192, 1024)),      # main + reduce kernels
+    "skinny128": ("d128x128_n3", "gemm_decode_kernel_skinny128_skinny64.md", (73797, 8210), (16384, 2048)),   # main + reduce kernels
 }
+MEASURED_TRAFFIC_BYTES = {w: (cfg, (sum(f) * FETCH_SCALE + sum(wr) * WRITE_SCALE) * 1024)
+                          for w, (cfg, _, f, wr) in MEASURED_TRAFFIC_KIB.items()}
+# The eight shapes of the benchmark definition, in its order: every run of the headline workload
+# also times the other seven (after the headline's timed region) and reports them as `configs`.
+BASELINE_WORKLOADS = ("square512", "square8192", "mlp_up", "mlp_down", "skinny16", "skinny64", "skinny128", "unaligned")
+
+
+def bound_of(M: int, N: int, K: int) -> str:
+    """What the shape is priced against: the bf16 MFMA peak, the HBM peak, or neither -- 512^3 is
+    0.2 us of either and a few microseconds of launch and pipeline latency (reported as it is)."""
+    flops, nbytes = 2.0 * M * N * K, 2.0 * (M * K + N * K + M * N)
+    if flops / (PEAK_BF16_TFLOPS * 1e12) < 1e-6 and nbytes / (PEAK_HBM_GBS * 1e9) < 1e-6:
+        return "launch"
+    return "hbm" if flops / nbytes < PEAK_BF16_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9) else "mfma"
 
 
 def make_inputs(orc, M, N, K, fill, seed=69):
@@ -97,6 +117,56 @@ def cpu_baseline(orc, A, B, budget_tiles: int) -> dict:
             "sample": f"{len(tiles)} of {total_tiles} 64x64 output tiles, full K={K}, "
                       f"reference loop order, {dt:.1f} s; whole problem extrapolates to "
                       f"{dt * total_tiles / len(tiles):.0f} s"}
+
+
+def time_workload(mi, orc, name: str, launches: int, check_tiles: int) -> dict:
+    """One row of `configs`: the library's own kernel choice on one benchmark shape, a short
+    settle, then `launches` back-to-back launches between two HIP events on the launch stream
+    (B rotated through three copies where HBM binds, so that the memory-side cache does not
+    serve it), and the tolerance check of the last result on a sample of 64x64 tiles."""
+    M, N, K, fill = WORKLOADS[name]
+    A, B = make_inputs(orc, M, N, K, fill)
+    bound = bound_of(M, N, K)
+    dA = mi.DeviceBuffer.from_numpy(A)
+    dBs = [mi.DeviceBuffer.from_numpy(B) for _ in range(3 if bound == "hbm" else 1)]
+    dC = mi.DeviceBuffer(M * N * 2)
+    cfg = mi.select_config(M, N, K)
+    params = [mi.GemmParams(M, N, K, dA, dB, dC) for dB in dBs]
+    t_end = time.perf_counter() + 0.1
+    while time.perf_counter() < t_end:
+        for i in range(8):
+            mi.gpu_gemm(params[i % len(params)], config=cfg)
+        mi.synchronize()
+    timer = mi.GPUTimer()
+    best = None
+    for _ in range(2):
+        timer.tick()
+        for i in range(launches):
+            mi.gpu_gemm(params[i % len(params)], config=cfg)
+        timer.tick()
+        mi.synchronize()
+        ms = timer.report_last_ms() / launches
+        best = ms if best is None or ms < best else best
+    violations = None
+    if check_tiles > 0:
+        C = dC.to_numpy((M, N), np.uint16)
+        tiles = orc.sample_tiles(M, N, check_tiles)
+        ref = orc.reference_cpu_gemm(A, B, tiles=tiles)
+        violations = orc.check_tolerance(C, ref, K, orc.max_abs(A), orc.max_abs(B), tiles=tiles)["violations"]
+    for b in [dA, dC, *dBs]:
+        b.free()
+    tflops = 2.0 * M * N * K / (best * 1e-3) / 1e12
+    gbs = 2.0 * (M * K + N * K + M * N) / (best * 1e-3) / 1e9
+    row = {"workload": name, "M": M, "N": N, "K": K, "kernel_config": mi.config_name(cfg),
+           "us_per_launch": best * 1e3, "launches": launches, "bound": bound, "tflops": tflops, "gbs_algorithmic": gbs}
+    if bound == "mfma":
+        row.update(achieved=tflops, unit="TFLOP/s", peak=PEAK_BF16_TFLOPS, frac=tflops / PEAK_BF16_TFLOPS)
+    elif bound == "hbm":
+        row.update(achieved=gbs, unit="GB/s", peak=PEAK_HBM_GBS, frac=gbs / PEAK_HBM_GBS)
+    else:       # launch latency: no roofline fraction is claimed
+        row.update(achieved=best * 1e3, unit="us", peak=None, frac=None)
+    row["tolerance_violations"] = violations
+    return row
 
 
 def sclk_under_load(launch_batch, sync) -> float | None:
@@ -196,6 +266,8 @@ def main() -> int:
                     help="do not sample the shader clock under load after the timed region")
     ap.add_argument("--no-ceiling", dest="ceiling", action="store_false",
                     help="do not run the MFMA-only loop (same-box ceiling) and the power sampling after the timed region")
+    ap.add_argument("--no-configs", dest="configs", action="store_false",
+                    help="headline workload only: do not time the other seven benchmark shapes after it")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain device-to-device copy of 256 MiB (a kernel of known HBM "
                          "traffic, for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
@@ -219,8 +291,8 @@ def main() -> int:
     A, B = make_inputs(orc, M, N, K, fill)
     flops = 2.0 * M * N * K
     algo_bytes = 2.0 * (M * K + N * K + M * N)
-    ridge = PEAK_BF16_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9)
-    hbm_bound = flops / algo_bytes < ridge
+    bound = bound_of(M, N, K)
+    hbm_bound = bound == "hbm"
     dA = mi.DeviceBuffer.from_numpy(A)
     # HBM-bound shapes: B (128 MiB) would otherwise be served by the 256 MB memory-side
     # cache on every launch after the first; rotate three copies so each launch reads HBM.
@@ -280,13 +352,15 @@ def main() -> int:
 
     tflops = flops / (ms_per_step * 1e-3) / 1e12
     gbs = algo_bytes / (ms_per_step * 1e-3) / 1e9
-    if not hbm_bound:
+    if bound == "mfma":
         roof = {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                 "frac": tflops / PEAK_BF16_TFLOPS}
-    else:
+    elif bound == "hbm":
         roof = {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                 "frac": gbs / PEAK_HBM_GBS}
-    if not hbm_bound and a.ceiling:
+    else:       # 512^3: launch and pipeline latency; neither roofline says anything about it
+        roof = {"bound": "launch", "achieved": ms_per_step * 1e3, "peak": None, "unit": "us", "frac": None}
+    if bound == "mfma" and a.ceiling:
         # the same-box yardstick: a slow box (they differ by +-6 % in the clock they sustain) moves
         # `achieved` and `ceiling_same_box` together, a kernel change moves only the first
         ceiling = mfma_ceiling_same_box(fill)
@@ -298,6 +372,27 @@ def main() -> int:
     roof["avg_launch_us"] = ms_per_step * 1e3
 
     cpu = cpu_baseline(orc, A, B, a.cpu_tiles) if a.cpu_tiles > 0 else None
+
+    # the other benchmark shapes, with the library's own kernel choice, in the same run (not
+    # under a profiler, where the run is about one kernel)
+    configs = None
+    if a.configs and a.workload == "square8192" and a.config is None and not _under_profiler():
+        for b in [dA, dC, *dBs]:
+            b.free()
+        configs = []
+        for name in BASELINE_WORKLOADS:
+            if name == a.workload:
+                row = {"workload": name, "M": M, "N": N, "K": K, "kernel_config": mi.config_name(cfg),
+                       "us_per_launch": ms_per_step * 1e3, "launches": a.steps, "bound": bound, "tflops": tflops,
+                       "gbs_algorithmic": gbs, "achieved": roof["achieved"], "unit": roof["unit"], "peak": roof["peak"],
+                       "frac": roof["frac"], "tolerance_violations": violations}
+            else:
+                # about 30 ms of launches per timed batch, 20 to 200 of them (estimated at half the peak rate)
+                Mw, Nw, Kw, _ = WORKLOADS[name]
+                est_us = max(2.0 * Mw * Nw * Kw / 1.25e15, 2.0 * (Mw * Kw + Nw * Kw + Mw * Nw) / 4e12) * 1e6
+                launches = int(min(200, max(20, 30000.0 / est_us)))
+                row = time_workload(mi, orc, name, launches, min(a.check_tiles, 64 if est_us < 200 else 16))
+            configs.append(row)
 
     out = {
         # the headline metric is quoted on square8192; the other workloads are labelled as what they are
@@ -318,8 +413,11 @@ def main() -> int:
         "roofline": roof,
         "cpu_baseline": cpu,
     }
+    if configs is not None:
+        out["configs"] = configs
     print(json.dumps(out))
-    return 0 if not violations else 1
+    bad = bool(violations) or any(r["tolerance_violations"] for r in (configs or []))
+    return 1 if bad else 0
 
 
 if __name__ == "__main__":

@@ -383,6 +383,16 @@ def test_bench_tables_are_well_formed(mi):
         assert name in bench.WORKLOADS                   # the BASELINE configurations
     for name, (config, nbytes) in bench.MEASURED_TRAFFIC_BYTES.items():
         assert name in bench.WORKLOADS and mi.find_config(config) >= 0 and nbytes > 0, name
+    # every traffic figure is the one the profile it cites shows (thousands separated by a space there)
+    for name, (config, profile, fetch, write) in bench.MEASURED_TRAFFIC_KIB.items():
+        text = (ROOT / "profiles" / profile).read_text()
+        for kib in (*fetch, *write):
+            assert f"{kib:,}".replace(",", " ") in text or str(kib) in text, f"{name}: {kib} KiB is not in profiles/{profile}"
+        assert f"`{config}`" in text or config in text, f"{name}: profiles/{profile} is not about {config}"
+    assert set(bench.BASELINE_WORKLOADS) <= set(bench.WORKLOADS) and len(bench.BASELINE_WORKLOADS) == 8
+    assert bench.bound_of(512, 512, 512) == "launch" and bench.bound_of(8192, 8192, 8192) == "mfma"
+    assert bench.bound_of(16, 8192, 8192) == "hbm" and bench.bound_of(128, 8192, 8192) == "hbm"
+    assert bench.bound_of(4095, 6143, 3073) == "mfma" and bench.bound_of(8192, 8192, 28672) == "mfma"
     out = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"], capture_output=True, text=True, cwd=ROOT)
     assert out.returncode == 2 and "ONE GPU" in out.stderr
 
