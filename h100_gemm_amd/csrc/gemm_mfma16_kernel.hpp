@@ -97,11 +97,18 @@ __device__ __forceinline__ f32x4_t mfma_16x16x32(u32x4_t a, u32x4_t b, f32x4_t c
 // that the plain kernel's registers and epilogue are untouched by it (a run-time branch to a
 // third epilogue made the 256-accumulator kernel spill in its last K step and epilogue).
 //
-// ABLATE (measurement aid, harness/gemm_power.hip; 0 in the library): parts of the K loop
-// compiled out so that their share of cycles and of power can be read off -- bit 0: no
-// global -> LDS loads after the prologue, bit 1: no LDS fragment reads in the loop, bit 2: no
-// barriers.  The results of such a kernel are meaningless.
+// Only when the header is compiled with -DMI_GEMM_ABLATE (harness/gemm_power.hip does, the
+// library does not) the kernel takes a fourth parameter ABLATE that compiles parts of the K
+// loop out, so that their share of cycles and of power can be read off -- bit 0: no global ->
+// LDS loads after the prologue, bit 1: no LDS fragment reads in the loop, bit 2: no barriers.
+// The results of such a kernel are meaningless.  In the library's build MI_ABLATED is `false`.
+#ifdef MI_GEMM_ABLATE
+#define MI_ABLATED(bits) ((ABLATE & (bits)) != 0)
 template <class Cfg, bool TRACE = false, bool SPLITK = false, int ABLATE = 0>
+#else
+#define MI_ABLATED(bits) false
+template <class Cfg, bool TRACE = false, bool SPLITK = false>
+#endif
 __global__ void __launch_bounds__(Cfg::NT)
 __attribute__((amdgpu_waves_per_eu(Cfg::WAVES_PER_EU, Cfg::WAVES_PER_EU)))
 gemm_mfma16_kernel(const GemmArgs p) {
@@ -219,7 +226,7 @@ gemm_mfma16_kernel(const GemmArgs p) {
                      :: "v"(voff), "s"(rsrc), "s"(soff), "n"(decltype(imm_c)::value) : "memory");
     };
     auto dma_one = [&](int kt, int stage, int d) __attribute__((always_inline)) {
-        if constexpr ((ABLATE & 1) != 0) { if (kt >= 2) return; }
+        if constexpr (MI_ABLATED(1)) { if (kt >= 2) return; }
         const uint32_t kb = (uint32_t)kt * (BK * 2);
         if constexpr (GROUPED) {
             if (d < LA) {
@@ -314,9 +321,9 @@ gemm_mfma16_kernel(const GemmArgs p) {
         acc[i][j] = mfma_16x16x32<DT>(fb[buf][j], fa[buf][i], acc[i][j]);
     };
     // fragment r of a slice in the order the MFMAs first need them: A0, B0..B(NI-1), A1..
-    bool in_loop = false;      // ABLATE bit 1: fragment reads only before the K loop
+    [[maybe_unused]] bool in_loop = false;      // (ablation bit 1: fragment reads only before the K loop)
     auto read_one = [&](int stage, int ks, int buf, int r) __attribute__((always_inline)) {
-        if constexpr ((ABLATE & 2) != 0) { if (in_loop) return; }
+        if constexpr (MI_ABLATED(2)) { if (in_loop) return; }
         if (r == 0 || r > NI) {
             const int i = r == 0 ? 0 : r - NI;
             fa[buf][i] = *(const u32x4_t*)(lds + stage * A_STAGE + a_wave + i * 2048 + rd_off[ks]);
@@ -373,7 +380,7 @@ gemm_mfma16_kernel(const GemmArgs p) {
             if constexpr (Cfg::DRAIN && has2) {
                 // every wave holds its slice-1 fragments: stage `cur` may be overwritten
                 if (idx == Cfg::SA) {
-                    if constexpr ((ABLATE & 4) != 0) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    if constexpr (MI_ABLATED(4)) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                     else asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
                 }
             }
@@ -390,7 +397,7 @@ gemm_mfma16_kernel(const GemmArgs p) {
                     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
                 fix_tail(kt + 1, nxt);
                 asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            } else if constexpr ((ABLATE & 4) != 0) {
+            } else if constexpr (MI_ABLATED(4)) {
                 asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
             } else if constexpr (Cfg::DRAIN && has2) {
                 asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" :: "n"(Cfg::D0) : "memory");
@@ -409,7 +416,7 @@ gemm_mfma16_kernel(const GemmArgs p) {
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    if constexpr ((ABLATE & 2) != 0) {      // both fragment buffers hold real operand data
+    if constexpr (MI_ABLATED(2)) {      // both fragment buffers hold real operand data
 #pragma unroll
         for (int r = 0; r < NFR; ++r) read_one(0, 1, 1, r);
     }

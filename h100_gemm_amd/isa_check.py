@@ -66,7 +66,7 @@ def check_no_scratch(unit: str, text: str) -> int:
     """The aligned, untraced 16x16x32 kernels of a unit use no scratch memory.  Returns how
     many kernel descriptors were checked."""
     found = re.findall(r"\.amdhsa_kernel (\S+).*?\.amdhsa_private_segment_fixed_size (\d+)", text, flags=re.S)
-    # Mfma16Config<..., EDGE, OCC, KG>, TRACE, SPLITK[, ABLATE]: "...ELb<EDGE>ELi<OCC>ELi<KG>EEELb<TRACE>ELb<SPLITK>..."
+    # Mfma16Config<..., EDGE, OCC, KG>, TRACE, SPLITK: "...ELb<EDGE>ELi<OCC>ELi<KG>EEELb<TRACE>ELb<SPLITK>..."
     aligned = [(n, int(sz)) for n, sz in found if re.search(r"Mfma16ConfigI\w*?ELb0ELi\d+ELi\d+EEELb0ELb[01]", n)]
     if not aligned:
         raise IsaCheckError(f"{unit}: no aligned 16x16x32 kernel found among {[n for n, _ in found]}")

@@ -85,7 +85,7 @@ def test_the_checks_reject_what_they_are_there_for():
         isa_check.check_m0("bad", KERNEL.format(body=GOOD.replace("	s_mov_b32 m0, s8\n	s_nop 0\n", ""), scratch=0))
     with pytest.raises(isa_check.IsaCheckError, match="kernels found"):
         isa_check.check_m0("empty", "no kernels here", need_kernels=1)
-    spilled = KERNEL.replace("_ZN2mi4testE", "_ZN2mi18gemm_mfma16_kernelINS_12Mfma16ConfigILi256ELi256ELi2ELi2ELi4ELi0ELi3ELb0ELi1ELi1EEELb0ELb0ELi0EEEvNS_8GemmArgsE")
+    spilled = KERNEL.replace("_ZN2mi4testE", "_ZN2mi18gemm_mfma16_kernelINS_12Mfma16ConfigILi256ELi256ELi2ELi2ELi4ELi0ELi3ELb0ELi1ELi1EEELb0ELb0EEEvNS_8GemmArgsE")
     assert isa_check.check_no_scratch("ok", spilled.format(body=GOOD, scratch=0)) == 1
     with pytest.raises(isa_check.IsaCheckError, match="scratch"):
         isa_check.check_no_scratch("bad", spilled.format(body=GOOD, scratch=64))
