@@ -104,6 +104,10 @@ def _check_unit(src: Path, obj: Path) -> None:
     if cfg["KIND"] == "mfma16" and cfg.get("EFF"):
         isa_check.check_no_scratch(src.name, text)
     isa_check.check_lds_bytes(src.name, text, kc.lds_bytes(cfg))
+    # registers with an asm-issued load in flight are left alone (the decode kernels' ring of A fragments)
+    n = isa_check.check_inflight(src.name, text)
+    if cfg["KIND"] == "decode" and n == 0:
+        raise RuntimeError(f"{src.name}: the decode kernel's asm loads into registers were not found in the assembly text")
 
 
 def _compile(src: Path, force: bool) -> Path:

@@ -135,14 +135,25 @@ gemm_decode_kernel(const DecodeArgs p) {
     int issued = 0;
     // A fragments arrive through inline asm like the B rows, so that every wait on `vmcnt` in
     // this kernel is an explicit one (the compiler, which cannot see the direct-to-LDS loads,
-    // would otherwise wait for too many).  A register set is only read after wait_slab(), which
-    // takes it as an in/out operand: nothing that uses it can be moved above the wait.
+    // would otherwise wait for too many).
+    // INVARIANT: between the asm statement that loads into a register of `areg` and the
+    // wait_slab() that retires that load, no instruction reads or writes that register.  Two
+    // things hold it up.  In the source, a register set is an in/out operand of every asm
+    // statement that concerns it -- the loads (so a set is live from its first load to the
+    // kernel's last wait, whether or not a later slab still reads it: it is never a dead value
+    // whose registers the allocator may hand out) and the waits (so nothing that uses a set can
+    // be moved above the wait that retires its loads) -- and only MFMAs behind such a wait read
+    // it.  In the build, since the source cannot forbid the allocator to copy or move a live
+    // value, isa_check.check_inflight follows the generated code of this kernel and refuses to
+    // link when any instruction touches a register with one of these loads still in flight.
     u32x4_t areg[NS][LA];
-    auto load_a = [](__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff, auto imm_c) __attribute__((always_inline)) {
-        u32x4_t v;
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+#pragma unroll
+        for (int i = 0; i < LA; ++i) areg[s][i] = u32x4_t{0u, 0u, 0u, 0u};
+    auto load_a = [](u32x4_t& dst, __amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff, auto imm_c) __attribute__((always_inline)) {
         asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:%4"
-                     : "=v"(v) : "v"(voff), "s"(rsrc), "s"(soff), "n"(decltype(imm_c)::value) : "memory");
-        return v;
+                     : "+v"(dst) : "v"(voff), "s"(rsrc), "s"(soff), "n"(decltype(imm_c)::value) : "memory");
     };
     // A request = the L loads of one slab (LA fragment loads of A, LB direct-to-LDS loads of B),
     // issued piece by piece so that they can be dealt out between the MFMAs of a slab.
@@ -160,7 +171,7 @@ gemm_decode_kernel(const DecodeArgs p) {
         constexpr int s = decltype(stage_c)::value;
         constexpr int pc = decltype(piece_c)::value;
         if constexpr (pc < LA) {
-            areg[s][pc] = load_a(ra_req, voffA[pc / 2], kb_req, std::integral_constant<int, (pc & 1) * 64>{});
+            load_a(areg[s][pc], ra_req, voffA[pc / 2], kb_req, std::integral_constant<int, (pc & 1) * 64>{});
         } else {
             constexpr int i = pc - LA;
             dma(rb_req, voffB[i], kb_req, lds_base + (uint32_t)(s * STAGE + (wave + i * 4) * 1024));
@@ -199,9 +210,7 @@ gemm_decode_kernel(const DecodeArgs p) {
     // they have for every wave, and every wave is done with the stage before it, which the
     // request for slab t + NS - 1 then refills.  TAIL >= 0 marks the last slabs of the walk,
     // TAIL-th after the requests have stopped: nothing is requested any more (it would lie
-    // past the split's last slab) and the wait counts down.  The requests have to stop there:
-    // a register set that no later slab reads is dead to the compiler, which would hand its
-    // registers to something else while the loads into them are still on their way.
+    // past the split's last slab) and the wait counts down.
     auto slab = [&](auto stage_c, auto tail_c) __attribute__((always_inline)) {
         constexpr int s = decltype(stage_c)::value;
         constexpr int TAIL = decltype(tail_c)::value;
@@ -247,8 +256,8 @@ gemm_decode_kernel(const DecodeArgs p) {
     });
     // Requests past this split's last slab (empty descriptor: they fetch nothing, but zeros
     // still arrive in their registers and LDS stages) may be outstanding.  Every A register
-    // set stays live up to this wait, whichever slabs the tail ran, so that the compiler
-    // cannot give a register with a load still on its way to anything else.
+    // set is an operand of the statement behind this wait, whichever slabs the tail ran: the
+    // end of the live range that the invariant above speaks of.
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     auto keep = [](u32x4_t (&a)[LA]) __attribute__((always_inline)) {
         if constexpr (LA == 2) asm volatile("" : "+v"(a[0]), "+v"(a[1]));

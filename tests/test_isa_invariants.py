@@ -89,3 +89,46 @@ def test_the_checks_reject_what_they_are_there_for():
     assert isa_check.check_no_scratch("ok", spilled.format(body=GOOD, scratch=0)) == 1
     with pytest.raises(isa_check.IsaCheckError, match="scratch"):
         isa_check.check_no_scratch("bad", spilled.format(body=GOOD, scratch=64))
+
+
+INFLIGHT = """	;;#ASMSTART
+	buffer_load_dwordx4 v[10:13], v1, s[0:3], s9 offen
+	;;#ASMEND
+	;;#ASMSTART
+	s_mov_b32 m0, s8
+	s_nop 0
+	buffer_load_dwordx4 v2, s[0:3], s9 offen lds
+	;;#ASMEND
+{between}
+	;;#ASMSTART
+	s_waitcnt vmcnt({n}) lgkmcnt(0)
+	s_barrier
+	;;#ASMEND
+	v_mfma_f32_16x16x32_bf16 a[0:3], v[10:13], v[6:9], a[0:3]"""
+
+
+def test_registers_with_an_asm_load_in_flight_are_left_alone():
+    """The decode kernels load A fragments into registers from their own asm statements; the
+    build follows those loads through the generated code."""
+    units = built_units(("decode",))
+    assert len(units) == 2
+    for name, c, text in units:
+        assert isa_check.check_inflight(name, text) >= 16, name
+    ok = KERNEL.format(body=INFLIGHT.format(between="	v_mov_b32_e32 v20, v5", n=1), scratch=0)
+    assert isa_check.check_inflight("ok", ok) == 1
+    # the allocator copying an in-flight register somewhere else
+    with pytest.raises(isa_check.IsaCheckError, match="touches"):
+        isa_check.check_inflight("bad", KERNEL.format(body=INFLIGHT.format(between="	v_mov_b32_e32 v20, v11", n=1), scratch=0))
+    # ... or handing it to another value
+    with pytest.raises(isa_check.IsaCheckError, match="touches"):
+        isa_check.check_inflight("bad", KERNEL.format(body=INFLIGHT.format(between="	v_add_u32_e32 v12, v1, v1", n=1), scratch=0))
+    # ... or spilling it
+    with pytest.raises(isa_check.IsaCheckError, match="uses|touches"):
+        isa_check.check_inflight("bad", KERNEL.format(body=INFLIGHT.format(between="	scratch_store_dwordx4 off, v[10:13], off offset:16", n=1), scratch=0))
+    # a wait that leaves the load in flight (two loads are younger than allowed to be outstanding)
+    with pytest.raises(isa_check.IsaCheckError, match="touches"):
+        isa_check.check_inflight("bad", KERNEL.format(body=INFLIGHT.format(between="", n=2), scratch=0))
+    # a loop whose next trip loads into a register before the wait of this trip has retired the last load
+    loop = ".LBB0_1:\n" + INFLIGHT.format(between="", n=2).replace("	v_mfma_f32_16x16x32_bf16 a[0:3], v[10:13]", "	v_mfma_f32_16x16x32_bf16 a[0:3], v[14:17]") + "\n	s_cbranch_scc1 .LBB0_1"
+    with pytest.raises(isa_check.IsaCheckError, match="still has a load in flight"):
+        isa_check.check_inflight("bad", KERNEL.format(body=loop, scratch=0))
