@@ -99,7 +99,8 @@ def _check_unit(src: Path, obj: Path) -> None:
     cfg = next((c for c in kc.CONFIGS if src.name == f"unit_{kc.config_name(c)}.hip"), None)
     if cfg is None:
         return                                  # not a kernel unit
-    # {bf16, fp16} x {aligned, predicated} x {plain, trace, split-K} for the 16x16x32 kernel
+    # {bf16, fp16} x {aligned, predicated} x {plain, trace} for the 16x16x32 kernel (and as many again
+    # with K cut over workgroups, where the config does not split K over groups of its waves)
     isa_check.check_m0(src.name, text, need_kernels=8 if cfg["KIND"] == "mfma16" else 1)
     if cfg["KIND"] == "mfma16" and cfg.get("EFF"):
         isa_check.check_no_scratch(src.name, text)

@@ -73,7 +73,8 @@ struct DecodeConfig {
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
 };
 
-template <class Cfg>
+// TRACE: the per-workgroup timing record (TraceRec) for launches that pass a trace buffer.
+template <class Cfg, bool TRACE = false>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 gemm_decode_kernel(const DecodeArgs p) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::NS, DT = Cfg::DT;
@@ -82,6 +83,8 @@ gemm_decode_kernel(const DecodeArgs p) {
     (void)BM;
 
     __shared__ __attribute__((aligned(128))) unsigned char lds[Cfg::LDS_BYTES];
+    TraceRec<TRACE> tr;
+    tr.begin();
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -215,11 +218,14 @@ gemm_decode_kernel(const DecodeArgs p) {
         constexpr int s = decltype(stage_c)::value;
         constexpr int TAIL = decltype(tail_c)::value;
         constexpr int sf = s == 0 ? NS - 1 : s - 1;
+        tr.wait_begin();
         if constexpr (TAIL < 0) {
             wait_slab(areg[s], std::integral_constant<int, NS - 2>{});
+            tr.wait_end();
             request_begin();
         } else {
             wait_slab(areg[s], std::integral_constant<int, NS - 2 - TAIL>{});
+            tr.wait_end();
         }
         const unsigned char* st = lds + s * STAGE;
         // Slice 0's B fragments, then slice 1's dealt out under the MFMAs of slice 0, and the
@@ -264,6 +270,7 @@ gemm_decode_kernel(const DecodeArgs p) {
         else asm volatile("" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]));
     };
     static_for<NS>([&](auto s_c) __attribute__((always_inline)) { keep(areg[decltype(s_c)::value]); });
+    tr.loop_end();
 
     // ---- epilogue: acc[i][j][e] of lane l is C[m][n], m = row0 + i*16 + (l & 15),
     //      n = col0 + j*16 + 4*(l >> 4) + e  (N % 4 == 0 is a launch precondition) ----
@@ -289,6 +296,7 @@ gemm_decode_kernel(const DecodeArgs p) {
                 }
             }
         }
+        tr.finish(p.DB, KT);
         return;
     }
     float* P = p.ws + (size_t)split * M * N;
@@ -301,12 +309,14 @@ gemm_decode_kernel(const DecodeArgs p) {
             if (m < M && n < N) *(f32x4_t*)(P + (size_t)m * N + n) = acc[i][j];
         }
     }
+    tr.finish(p.DB, KT);
 }
 
 template <class Cfg>
 hipError_t launch_decode_kernel(const DecodeArgs& a, hipStream_t stream) {
     dim3 grid((a.N + Cfg::BN - 1) / Cfg::BN, a.splits);
-    hipError_t e = launch_kernel(gemm_decode_kernel<Cfg>, grid, dim3(256), stream, a);
+    hipError_t e = a.DB ? launch_kernel(gemm_decode_kernel<Cfg, true>, grid, dim3(256), stream, a)
+                        : launch_kernel(gemm_decode_kernel<Cfg, false>, grid, dim3(256), stream, a);
     if (e != hipSuccess || a.splits == 1) return e;
     const size_t quads = ((size_t)a.M * a.N + 3) / 4;
     return launch_kernel(splitk_reduce_kernel<Cfg::DT>, dim3((unsigned)((quads + 255) / 256)), dim3(256), stream,

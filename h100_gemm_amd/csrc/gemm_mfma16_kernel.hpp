@@ -580,7 +580,7 @@ gemm_mfma16_kernel(const GemmArgs p) {
         if (p.DB != nullptr && tid == 0) {
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             tr_store = tr_now() - tr_store;
-            int* rec = p.DB + 6 * (size_t)blockIdx.x;
+            int* rec = p.DB + 6 * ((size_t)blockIdx.y * gridDim.x + blockIdx.x);      // (blockIdx.y: the piece of a split-K launch)
             rec[0] = (int)tr_wait;
             rec[1] = tr_cnt;
             rec[2] = (int)tr_loop;
@@ -813,9 +813,8 @@ template <class Cfg, bool TRACE = false>
 hipError_t launch_mfma16_kernel(const GemmArgs& args, hipStream_t stream) {
     const int grid = args.tiles_m * args.tiles_n;
     if (args.splits > 1) {
-        if constexpr (TRACE) return hipErrorInvalidValue;   // no trace records from split-K launches
         if constexpr (Cfg::KG == 1)
-            return launch_kernel(gemm_mfma16_kernel<Cfg, false, true>, dim3(grid, args.splits), dim3(Cfg::NT), stream, args);
+            return launch_kernel(gemm_mfma16_kernel<Cfg, TRACE, true>, dim3(grid, args.splits), dim3(Cfg::NT), stream, args);
         else
             return hipErrorInvalidValue;        // K is already split inside the workgroup
     }

@@ -48,12 +48,16 @@ struct StreamConfig {
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
 };
 
-template <class Cfg>
+// TRACE: the per-workgroup timing record (TraceRec; thread 0 is in wave 0, so the waits and the
+// K units are that wave's) for launches that pass a trace buffer.
+template <class Cfg, bool TRACE = false>
 __global__ void __launch_bounds__(256) gemm_stream_kernel(const DecodeArgs p) {
     constexpr int BM = Cfg::BM, NS = Cfg::NS, DT = Cfg::DT;
     constexpr int L = Cfg::L, STAGE = Cfg::STAGE, RING = Cfg::RING, MI = Cfg::MI;
 
     __shared__ __attribute__((aligned(128))) unsigned char lds[Cfg::LDS_BYTES];
+    TraceRec<TRACE> tr;
+    tr.begin();
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -133,7 +137,9 @@ __global__ void __launch_bounds__(256) gemm_stream_kernel(const DecodeArgs p) {
     int s = 0;
     for (int i = 0; i < cnt; ++i) {
         // slab i of this wave has landed; its predecessor's fragments are in registers
+        tr.wait_begin();
         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" :: "n"((NS - 2) * L) : "memory");
+        tr.wait_end();
         dma_slab(i + NS - 1, s == 0 ? NS - 1 : s - 1);
         const unsigned char* st = ring + s * STAGE;
         u32x4_t fa[MI][4], fb[4];
@@ -151,6 +157,7 @@ __global__ void __launch_bounds__(256) gemm_stream_kernel(const DecodeArgs p) {
     }
     // requests past K are still heading for the ring: drain before it is reused
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    tr.loop_end();
 
     // ---- add the four partial tiles in wave order, round, store ----
     // lane holds P[m][n .. n+3], m = 32a + (lane & 31), n = 8g + 4*(lane >> 5)
@@ -185,11 +192,13 @@ __global__ void __launch_bounds__(256) gemm_stream_kernel(const DecodeArgs p) {
             *(u32x2_t*)((unsigned char*)p.C + ((size_t)m * p.ldc + col0 + n) * 2) = w2;
         }
     }
+    tr.finish(p.DB, cnt);
 }
 
 template <class Cfg>
 hipError_t launch_stream_kernel(const DecodeArgs& a, hipStream_t stream) {
-    return launch_kernel(gemm_stream_kernel<Cfg>, dim3((a.N + 31) / 32), dim3(256), stream, a);
+    return a.DB ? launch_kernel(gemm_stream_kernel<Cfg, true>, dim3((a.N + 31) / 32), dim3(256), stream, a)
+                : launch_kernel(gemm_stream_kernel<Cfg, false>, dim3((a.N + 31) / 32), dim3(256), stream, a);
 }
 
 }  // namespace mi

@@ -106,8 +106,12 @@ struct WaveKConfig {
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
 };
 
-template <class Cfg>
+// TRACE: the per-workgroup timing record (TraceRec; thread 0 is in wave 0, so the waits and the
+// K units are that wave's) for launches that pass a trace buffer.
+template <class Cfg, bool TRACE = false>
 __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
+    TraceRec<TRACE> tr;
+    tr.begin();
     constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::NS, DT = Cfg::DT;
     constexpr int MI = Cfg::MI, NI = Cfg::NI, L = Cfg::L, STAGE = Cfg::STAGE;
     constexpr int PITCH = Cfg::PITCH, REGION = Cfg::REGION;
@@ -212,7 +216,9 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
     int s = 0;
     for (int u = 0; u < cnt; ++u) {
         // unit u of this wave has landed
+        tr.wait_begin();
         asm volatile("s_waitcnt vmcnt(%0)" :: "n"((NS - 1) * L) : "memory");
+        tr.wait_end();
         if (tail_elems != 0 && wave + 4 * u == KT - 1) {
             // the matrix's last unit ends inside a chunk: each lane looks after what it fetched
 #pragma unroll
@@ -244,6 +250,7 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
     // requests past this wave's last unit (empty descriptor: zeros) are still heading for
     // the ring: drain before the partial tile takes its place
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    tr.loop_end();
 
     // ---- add the four partial tiles in wave order, scale, round, store ----
     // acc[i][j][e] of lane l is P[m][n], m = i*16 + (l & 15), n = j*16 + 4*(l >> 4) + e
@@ -323,6 +330,7 @@ __global__ void __launch_bounds__(256) gemm_wavek_kernel(const DecodeArgs p) {
     else if ((K & 1) != 0) store_c(std::integral_constant<int, 4>{});
     else if (c_vec_ok) store_c(std::integral_constant<int, 1>{});
     else store_c(std::integral_constant<int, 3>{});
+    tr.finish(p.DB, cnt);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -360,8 +368,11 @@ struct SharedRingConfig {
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
 };
 
-template <class Cfg>
+// TRACE: the per-workgroup timing record (TraceRec) for launches that pass a trace buffer.
+template <class Cfg, bool TRACE = false>
 __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs p) {
+    TraceRec<TRACE> tr;
+    tr.begin();
     constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::NS, DT = Cfg::DT;
     constexpr int MI = Cfg::MI, NI = Cfg::NI, LW = Cfg::LW, STAGE = Cfg::STAGE;
     constexpr int TM = Cfg::TM, TN = Cfg::TN, PITCH = Cfg::PITCH;
@@ -501,6 +512,7 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
         constexpr bool TAIL = decltype(tail_c)::value;
         // this wave's loads of unit u + 1 have landed; after the barrier everyone's have, and
         // everyone has multiplied unit u - 1, whose stage takes the request NS - 1 units ahead
+        tr.wait_begin();
         if constexpr (TAIL) {
             asm volatile("s_waitcnt vmcnt(%0)" :: "n"((NS - 3) * LW) : "memory");
             fix_tail(s + 1 == NS ? 0 : s + 1);
@@ -509,6 +521,7 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
             asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"((NS - 3) * LW) : "memory");
             ++landed;
         }
+        tr.wait_end();
         request(s == 0 ? NS - 1 : s - 1, tail_c);
         read_unit(s + 1 == NS ? 0 : s + 1, fa[CUR ^ 1], fb[CUR ^ 1]);   // (past the last unit: zeros or stale rows, never multiplied)
         __builtin_amdgcn_sched_barrier(0);
@@ -546,6 +559,7 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
     // requests past the last unit (empty descriptor: zeros) are still heading for the ring, and
     // other waves may still be reading the last stage: drain and meet before C takes its place
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    tr.loop_end();
 
     // ---- the C tile through LDS as fp32, then scaled, rounded once and stored 8 bytes per lane ----
     // acc[i][j][e] of lane l is C[m][n], m = wm*TM + i*16 + (l & 15), n = wn*TN + j*16 + 4*(l >> 4) + e
@@ -618,6 +632,7 @@ __global__ void __launch_bounds__(256) gemm_shared_ring_kernel(const DecodeArgs 
     else if ((K & 1) != 0) store_c(std::integral_constant<int, 4>{});
     else if (c_vec_ok) store_c(std::integral_constant<int, 1>{});
     else store_c(std::integral_constant<int, 3>{});
+    tr.finish(p.DB, KT);
 }
 
 // the second launch of a split-K run: the pieces' sums added in order, scaled, rounded once
@@ -631,14 +646,16 @@ hipError_t launch_splitk_reduce(const DecodeArgs& a, hipStream_t stream) {
 template <class Cfg>
 hipError_t launch_shared_ring_kernel(const DecodeArgs& a, hipStream_t stream) {
     const int tiles = ((a.M + Cfg::BM - 1) / Cfg::BM) * ((a.N + Cfg::BN - 1) / Cfg::BN);
-    hipError_t e = launch_kernel(gemm_shared_ring_kernel<Cfg>, dim3(tiles, a.splits), dim3(256), stream, a);
+    hipError_t e = a.DB ? launch_kernel(gemm_shared_ring_kernel<Cfg, true>, dim3(tiles, a.splits), dim3(256), stream, a)
+                        : launch_kernel(gemm_shared_ring_kernel<Cfg, false>, dim3(tiles, a.splits), dim3(256), stream, a);
     return e != hipSuccess || a.splits == 1 ? e : launch_splitk_reduce<Cfg::DT>(a, stream);
 }
 
 template <class Cfg>
 hipError_t launch_wavek_kernel(const DecodeArgs& a, hipStream_t stream) {
     const int tiles = ((a.M + Cfg::BM - 1) / Cfg::BM) * ((a.N + Cfg::BN - 1) / Cfg::BN);
-    hipError_t e = launch_kernel(gemm_wavek_kernel<Cfg>, dim3(tiles, a.splits), dim3(256), stream, a);
+    hipError_t e = a.DB ? launch_kernel(gemm_wavek_kernel<Cfg, true>, dim3(tiles, a.splits), dim3(256), stream, a)
+                        : launch_kernel(gemm_wavek_kernel<Cfg, false>, dim3(tiles, a.splits), dim3(256), stream, a);
     return e != hipSuccess || a.splits == 1 ? e : launch_splitk_reduce<Cfg::DT>(a, stream);
 }
 

@@ -84,11 +84,11 @@ bool is_split_k_decode(int kind) { return kind == mi::KIND_DECODE; }
 // idle (small M x N, long K), the K range is cut into pieces of whole 128-deep steps, one
 // workgroup per (tile, piece); fp32 partials go to the workspace and splitk_reduce_kernel
 // adds them in order.  The piece count comes from the time model of the kernel table
-// (best_splits); the reduction's vector accesses need N % 4 == 0 and an 8-byte aligned C,
-// and a trace buffer has one record per tile, so those cases do not split.
+// (best_splits); the reduction's vector accesses need N % 4 == 0 and an 8-byte aligned C.
+// (A trace buffer changes nothing: every workgroup of a split launch writes its record.)
 // MI_GEMM_TILE_SPLITK=<n> forces a piece count (1 = never split; tuning aid).
-bool shape_is_splittable(int N, const void* C, const int* DB) {
-    return DB == nullptr && N % 4 == 0 && ((uintptr_t)C & 7u) == 0;
+bool shape_is_splittable(int N, const void* C) {
+    return N % 4 == 0 && ((uintptr_t)C & 7u) == 0;
 }
 
 int choose_tile_splits(const mi::KernelEntry& e, int M, int N, int K, bool splittable, bool ptr_aligned, int cus,
@@ -433,6 +433,13 @@ int rows_to_cut(int M, int N, int K, bool streamable, bool splittable, bool ptr_
     return memo.m1;
 }
 
+// Workgroups the main kernel of a launch has (the grid a trace buffer's records are indexed by).
+size_t launch_workgroups(const mi::KernelEntry& e, int M, int N, int splits) {
+    const size_t tiles_n = (size_t)(N + e.BN - 1) / e.BN;
+    if (e.kind == mi::KIND_STREAM || is_split_k_decode(e.kind)) return tiles_n * (size_t)splits;
+    return (size_t)((M + e.BM - 1) / e.BM) * tiles_n * (size_t)splits;
+}
+
 // One GEMM launch (two for split-K): argument checks, kernel choice, aligned / predicated twin.
 // `may_cut`: the automatic choice may run the shape as two GEMMs, the first rows and the rest
 // (rows_to_split_off in the kernel table); the parts themselves are not cut again.
@@ -441,9 +448,9 @@ int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const vo
     int rc = check_args(config, dtype, M, N, K, A, B, C);
     if (rc != MI_OK) return rc;
     const bool streamable = shape_is_streamable(M, N, K, A, B, C);
-    if (may_cut && config == MI_CONFIG_AUTO && DB == nullptr &&
+    if (may_cut && config == MI_CONFIG_AUTO &&
         tuned_config(M, N, K, streamable, shape_has_word_rows(K, A, B)) < 0) {       // (a tuned shape runs as tuned)
-        const int m1 = rows_to_cut(M, N, K, streamable, shape_is_splittable(N, C, DB),
+        const int m1 = rows_to_cut(M, N, K, streamable, shape_is_splittable(N, C),
                                    aligned16(A) && aligned16(B) && aligned16(C), shape_has_word_rows(K, A, B));
         if (m1 > 0) {
             // Both parts' workspace is settled before anything is launched: a part that could not
@@ -452,31 +459,31 @@ int run_gemm(int config, int dtype, int M, int N, int K, const void* A, const vo
             const void* A2 = (const unsigned char*)A + (size_t)m1 * K * 2;
             void* C2 = (unsigned char*)C + (size_t)m1 * N * 2;
             size_t need = 0;
+            size_t wgs_first = 0;            // workgroups of the first part: the second part's trace records follow theirs
             for (int part = 0; part < 2; ++part) {
                 const int Mp = part ? M - m1 : m1;
                 const void* Ap = part ? A2 : A;
                 const void* Cp = part ? C2 : C;
-                const Choice c = choose(config, Mp, N, K, shape_is_streamable(Mp, N, K, Ap, B, Cp), shape_is_splittable(N, Cp, nullptr),
+                const Choice c = choose(config, Mp, N, K, shape_is_streamable(Mp, N, K, Ap, B, Cp), shape_is_splittable(N, Cp),
                                         aligned16(Ap) && aligned16(B) && aligned16(Cp), shape_has_word_rows(K, Ap, B));
                 const size_t b = c.splits > 1 ? (size_t)c.splits * Mp * N * sizeof(float) : 0;
                 if (b > need) need = b;
+                if (part == 0) wgs_first = launch_workgroups(mi::kKernels[c.config], Mp, N, c.splits);
             }
             if (need > 0) {
                 float* unused = nullptr;
                 const int wrc = acquire_workspace(wsrc, need, (hipStream_t)stream, &unused);
                 if (wrc < 0) return wrc;
             }
-            rc = run_gemm(config, dtype, m1, N, K, A, B, C, nullptr, alpha, beta, stream, wsrc, false);
+            rc = run_gemm(config, dtype, m1, N, K, A, B, C, DB, alpha, beta, stream, wsrc, false);
             if (rc != MI_OK) return rc;
-            return run_gemm(config, dtype, M - m1, N, K, A2, B, C2, nullptr, alpha, beta, stream, wsrc, false);
+            return run_gemm(config, dtype, M - m1, N, K, A2, B, C2, DB ? DB + 6 * wgs_first : nullptr, alpha, beta, stream,
+                            wsrc, false);
         }
     }
-    // with a trace buffer the automatic choice stays with the kernels that fill it (the tiled
-    // ones); an explicitly requested decode or small-tile kernel runs and leaves it untouched
-    const Choice choice = choose(config, M, N, K, streamable && !(config == MI_CONFIG_AUTO && DB),
-                                 shape_is_splittable(N, C, DB),
-                                 aligned16(A) && aligned16(B) && aligned16(C),
-                                 shape_has_word_rows(K, A, B) && !(config == MI_CONFIG_AUTO && DB));
+    // (a trace buffer does not change the choice: every kernel family writes the records)
+    const Choice choice = choose(config, M, N, K, streamable, shape_is_splittable(N, C),
+                                 aligned16(A) && aligned16(B) && aligned16(C), shape_has_word_rows(K, A, B));
     config = choice.config;
     const mi::KernelEntry& e = mi::kKernels[config];
 
@@ -664,12 +671,23 @@ int mi_gemm_row_cut(int dtype, int M, int N, int K) {
 int mi_gemm_tuned_entries(void) { return (int)tuned_entries().size(); }
 
 size_t mi_gemm_trace_words(int M, int N, int K) {
-    // enough for whichever kernel configuration ends up running the shape
-    size_t grid = 0;
-    for (int c = 0; c < mi::kNumKernels; ++c) {
-        const size_t g = (size_t)mi_gemm_config_grid(c, M, N, K);
-        if (g > grid) grid = g;
-    }
+    // enough for whichever kernel configuration ends up running the shape -- or its two
+    // parts, one after the other, where the automatic choice cuts the shape's rows
+    auto largest = [&](int rows) {
+        size_t grid = 0;
+        for (int c = 0; c < mi::kNumKernels; ++c) {
+            const size_t g = (size_t)mi_gemm_config_grid(c, rows, N, K);
+            if (g > grid) grid = g;
+        }
+        return grid;
+    };
+    size_t grid = largest(M);
+    if (shape_in_range(M, N, K))
+        for (int flags = 0; flags < 16; ++flags) {
+            const int m1 = rows_to_cut(M, N, K, (flags & 1) != 0 && N % 4 == 0 && K % 64 == 0, (flags & 2) != 0 && N % 4 == 0,
+                                       (flags & 4) != 0, (flags & 8) != 0);
+            if (m1 > 0 && largest(m1) + largest(M - m1) > grid) grid = largest(m1) + largest(M - m1);
+        }
     return grid * 6 + 1;
 }
 

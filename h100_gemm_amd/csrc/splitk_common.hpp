@@ -25,6 +25,39 @@ struct DecodeArgs {
     int splits;           // <= K / 64
     float alpha = 1.0f;   // C = (CType)(acc * alpha + beta), applied where the sum over K is
     float beta = 0.0f;    // complete
+    int* DB = nullptr;    // optional trace buffer: one record of six ints per workgroup
+};
+
+// The per-workgroup timing record of the trace buffer `DB` of runKernel's signature, in the
+// format its harness parses (matmul_h100_optimal.cu:182-198): {sumLoad, cntLoad, sumCompute,
+// cntCompute, sumStore, cntStore} = {cycles thread 0 spent waiting for loads (and at the
+// barriers behind those waits), number of such waits, cycles from the kernel's start to the end
+// of its K loop, K units it multiplied, cycles from there to its last store, 1}.  Workgroup
+// (x, y) of a grid writes record y * gridDim.x + x.  With ON = false every member is empty.
+template <bool ON>
+struct TraceRec {
+    long long wait = 0, t0 = 0, loop = 0, store = 0;
+    int cnt = 0;
+    static __device__ __forceinline__ long long now() { return (long long)__builtin_readcyclecounter(); }
+    __device__ __forceinline__ void begin() { if constexpr (ON) loop = now(); }
+    __device__ __forceinline__ void wait_begin() { if constexpr (ON) t0 = now(); }
+    __device__ __forceinline__ void wait_end() { if constexpr (ON) { wait += now() - t0; ++cnt; } }
+    __device__ __forceinline__ void loop_end() { if constexpr (ON) { store = now(); loop = store - loop; } }
+    __device__ __forceinline__ void finish(int* DB, int units) {
+        if constexpr (ON) {
+            if (DB != nullptr && threadIdx.x == 0) {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                store = now() - store;
+                int* rec = DB + 6 * ((size_t)blockIdx.y * gridDim.x + blockIdx.x);
+                rec[0] = (int)wait;
+                rec[1] = cnt;
+                rec[2] = (int)loop;
+                rec[3] = units;
+                rec[4] = (int)store;
+                rec[5] = 1;
+            }
+        }
+    }
 };
 
 // C[m][n] = round(alpha * (sum over splits, in split order, of ws[s][m][n]) + beta); 4 elements per thread.

@@ -185,7 +185,12 @@ int mi_gemm_config_lds_bytes(int config);
 
 /* Number of `int` words a DB trace buffer must hold for this shape so that the kernel's
  * per-workgroup records plus the terminating sentinel fit (the harness of
- * matmul_h100_optimal.cu:132-139 allocates 8192*128 ints). */
+ * matmul_h100_optimal.cu:132-139 allocates 8192*128 ints).  Every kernel family writes the
+ * records -- six ints per workgroup, {cycles waiting for loads, waits, cycles to the end of the
+ * K loop, K units, cycles of the stores, 1}, in the format matmul_h100_optimal.cu:182-198
+ * parses -- so a trace buffer never changes which kernel MI_CONFIG_AUTO runs: a split-K launch
+ * writes one record per (tile, piece), workgroup (x, y) at record y * gridDim.x + x, and a shape
+ * that runs as two GEMMs (mi_gemm_row_cut) writes the first part's records, then the second's. */
 size_t mi_gemm_trace_words(int M, int N, int K);
 
 /* ---- thin HIP layer used by the C++ harness ------------------------------------------

@@ -881,39 +881,69 @@ def test_reference_gpu_gemm_is_bit_identical_to_the_oracle(mi, orc):
 # ------------------------------------------------------------------ trace buffer ------
 
 def test_db_trace_records(mi, orc):
+    """The DB buffer of runKernel's signature (matmul_h100_optimal.cu:32,132-139,182-198): every
+    kernel family writes one record {sumLoad, cntLoad, sumCompute, cntCompute, sumStore,
+    cntStore} per workgroup, a trace buffer never changes which kernel the automatic choice
+    runs, and results are the same with and without it."""
     from h100_gemm_amd import kernel_configs as kc
-    M = N = K = 1024
-    A, B = make_inputs(orc, M, N, K, "int")
-    d = Dev(mi, A, B, M, N)
-    words = mi._lib.load().mi_gemm_trace_words(M, N, K)
-    dDB = mi.DeviceBuffer(words * 4)
+    L = mi._lib.load()
 
-    def records(config):
+    def records(M, N, K, config, fill="int"):
+        A, B = make_inputs(orc, M, N, K, fill)
+        d = Dev(mi, A, B, M, N)
+        plain = d.run(K, config).copy()
+        words = L.mi_gemm_trace_words(M, N, K)
+        dDB = mi.DeviceBuffer(words * 4)
         dDB.fill_bytes(0xFF)
+        d.dC.fill_bytes(0xFF)
         C = d.run(K, config, DB=dDB)
-        assert (C == orc.reference_cpu_gemm(A, B)).all()        # tracing must not change results
+        assert (C == plain).all(), f"{M}x{N}x{K}: tracing changed {int((C != plain).sum())} elements"
+        if fill == "int":
+            assert (C == orc.reference_cpu_gemm(A, B)).all()
         db = dDB.to_numpy((words,), np.int32)
         n = 0
         while n + 5 < words and db[n] != -1:
             n += 6
-        assert db[n] == -1
-        return db[:n].reshape(-1, 6)
+        assert db[n] == -1 and (db[n:] == -1).all()         # the records are contiguous, the sentinel untouched
+        for b in (d.dA, d.dB, d.dC, dDB):
+            b.free()
+        rec = db[:n].reshape(-1, 6)
+        assert (rec[:, 5] == 1).all() and (rec[:, 2] > 0).all() and (rec[:, 4] > 0).all()
+        assert (rec[:, 0] >= 0).all() and (rec[:, 0] < rec[:, 2]).all() and (rec[:, 1] > 0).all()
+        return rec
 
+    # a tiled kernel by name: one record per tile, K / 64 steps each
     cfg = mi.find_config("m128x128_w2x2_g4_b1_o2")
-    rec = records(cfg)
-    assert len(rec) == mi.config_grid(cfg, M, N, K) == 64
-    assert (rec[:, 3] == K // 64).all() and (rec[:, 5] == 1).all()
-    assert (rec[:, 2] > 0).all() and (rec[:, 0] >= 0).all() and (rec[:, 0] < rec[:, 2]).all()
-    # the automatic choice for this shape is a small-tile kernel, which keeps no records: with
-    # a trace buffer it stays with the tiled kernels
-    assert kc.CONFIGS[mi.select_config(M, N, K)]["KIND"] == "wavek"
-    rec = records(mi.MI_CONFIG_AUTO)
-    tiled = [i for i, c in enumerate(kc.CONFIGS) if c["KIND"] == "mfma16" and c.get("EFF")]
-    assert len(rec) in {-(-M // kc.CONFIGS[i]["BM"]) * -(-N // kc.CONFIGS[i]["BN"]) for i in tiled}
-    # K steps per workgroup (per group of waves where a kernel splits K over two of them)
-    assert (rec[:, 3] == K // 64).all() or (rec[:, 3] == K // 128).all()
-    # asked for by name, the small-tile kernel runs and leaves the buffer untouched
-    assert len(records(mi.select_config(M, N, K))) == 0
+    rec = records(1024, 1024, 1024, cfg)
+    assert len(rec) == mi.config_grid(cfg, 1024, 1024, 1024) == 64 and (rec[:, 3] == 16).all()
+    # the automatic choice on the shapes of the benchmark's other kernel families: 512^3 (small
+    # tiles, K split over the waves: wave 0's units), 16 x 8192 x 8192 (single-pass decode: wave
+    # 0's slabs), 128 x 8192 x 8192 (split-K decode: a record per column tile and piece), and a
+    # mid-sized output on the shared-ring kernel
+    for (M, N, K), kind, units in [((512, 512, 512), "wavek", lambda c: 512 // 64 // 4),
+                                   ((16, 8192, 8192), "stream", lambda c: 8192 // 64 // 4),
+                                   ((128, 8192, 8192), "decode", lambda c: 8192 // 64 // 4),
+                                   ((1440, 1440, 1472), "wavek", lambda c: 1472 // 64)]:
+        auto = mi.select_config(M, N, K)
+        assert kc.CONFIGS[auto]["KIND"] == kind, (M, N, K, mi.config_name(auto))
+        rec = records(M, N, K, mi.MI_CONFIG_AUTO)
+        assert len(rec) == mi.config_grid(auto, M, N, K), (M, N, K, len(rec))
+        assert (rec[:, 3] == units(auto)).all(), (M, N, K, rec[:4])
+    # K cut over workgroups: the tiled split-K (256 x 8192 x 8192) and the small-tile kernels' (128 x 384 x 13376)
+    for M, N, K in [(256, 8192, 8192), (128, 384, 13376)]:
+        auto = mi.select_config(M, N, K)
+        grid = mi.config_grid(auto, M, N, K)
+        tiles = -(-M // kc.CONFIGS[auto]["BM"]) * -(-N // kc.CONFIGS[auto]["BN"])
+        assert grid > tiles and grid % tiles == 0                       # more than one piece per tile
+        rec = records(M, N, K, mi.MI_CONFIG_AUTO)
+        assert len(rec) == grid, (M, N, K, len(rec), grid)
+    # a shape that runs as two GEMMs: the first part's records, then the second part's
+    M, N, K = 7000, 7000, 4096
+    m1 = mi.row_cut(M, N, K)
+    assert m1 > 0
+    rec = records(M, N, K, mi.MI_CONFIG_AUTO, fill="uniform")
+    first, second = mi.select_config(m1, N, K), mi.select_config(M - m1, N, K)
+    assert len(rec) == mi.config_grid(first, m1, N, K) + mi.config_grid(second, M - m1, N, K)
 
 
 # --------------------------------------------------------------- C++ harness ----------
