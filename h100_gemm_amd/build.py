@@ -146,7 +146,7 @@ def build(jobs: int | None = None, force: bool = False, verbose: bool = True) ->
     return LIB
 
 
-# Two points of the tuner's search space, rendered from template/matmul_mi355x.hip.jinja and
+# Four points of the tuner's search space, rendered from template/matmul_mi355x.hip.jinja and
 # compiled as standalone `./test` programs -- the tuner's own flow (render -> hipcc -> run),
 # whose programs instantiate the kernels directly instead of going through the library's
 # dispatch.  Built here, where hipcc runs without a GPU, so that the GPU tests only run them.
@@ -154,6 +154,11 @@ TUNER_SAMPLES = PKG / "harness" / "tuner_samples"
 TUNER_SAMPLE_CONFIGS = [
     dict(KIND="mfma16", BM=256, BN=256, WM=2, WN=2, NS=4, SWZ=1, GROUP=4, DTL=1, EPI=1, DRAIN=3, OCC=1),
     dict(KIND="tile", BM=128, BN=128, WM=2, WN=2, NS=4, SWZ=1, GROUP=8, DTL=1, EPI=1, DRAIN=0, OCC=2),
+    # kinds whose LDS stage count the tuner sweeps: a split-K decode kernel with a ring of four
+    # slabs of B and a small-tile kernel with per-wave rings of three stages (neither depth is
+    # among the library's own configurations)
+    dict(KIND="decode", BM=128, BN=128, WM=2, WN=2, NS=4, GROUP=4, DRAIN=0, OCC=1, SHARED=0),
+    dict(KIND="wavek", BM=64, BN=64, WM=2, WN=2, NS=3, GROUP=4, DRAIN=0, OCC=1, SHARED=0),
 ]
 
 

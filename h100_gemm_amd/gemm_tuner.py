@@ -4,8 +4,9 @@ The counterpart of the reference's ``gemm_tuner.py`` (gemm_tuner.py:11-181), wit
 class, methods, control flow, failure handling and output files, retargeted from Hopper to
 CDNA4:
 
-* the search space is MFMA macro tile, wave grid, pipeline kind/depth, LDS swizzle, tile-order
-  group, load path and epilogue instead of cluster shape / block / TMA stages
+* the search space is MFMA macro tile, wave layout, pipeline kind and LDS stage count (of the
+  rings of the decode and small-tile kernels, where the depth is a free parameter), tile-order
+  group, occupancy and drain slot instead of cluster shape / block / TMA stages
   (gemm_tuner.py:17-24);
 * a configuration is rendered from ``template/matmul_mi355x.hip.jinja``, compiled with
   ``hipcc --offload-arch=gfx950`` (nvcc -arch=sm_90a there, gemm_tuner.py:46) and run as
@@ -76,20 +77,23 @@ class GemmTuner:
         # an explicit list of configurations instead of the grid below
         self.only = only
 
-        # Define parameter search space
+        # Define parameter search space: MFMA macro tile, wave layout and LDS stage count (what the
+        # reference sweeps as BLOCKM and STAGES, gemm_tuner.py:17-24), plus tile-order group,
+        # occupancy and the drain slot of the 16x16x32 kernel.  NS is a real parameter where the
+        # LDS ring's depth is one: the decode kinds and the small-tile kind (is_valid_configuration
+        # keeps one copy of every configuration it means nothing for, and the ring kinds of the
+        # tiled kernels exist with four stages only).
         self.param_space = {
-            'KIND': ['mfma16', 'ring', 'ring16', 'tile'],
-            'BM': [128, 192, 256],
-            'BN': [128, 192, 256],
+            'KIND': ['mfma16', 'ring', 'ring16', 'tile', 'stream', 'decode', 'wavek'],
+            'BM': [16, 32, 64, 96, 128, 192, 256],
+            'BN': [32, 64, 96, 128, 192, 256],
             'WM': [2, 4],
             'WN': [2, 4],
-            'NS': [4],
-            'SWZ': [1],
+            'NS': [4, 1, 2, 3, 5],
             'GROUP': [4, 8],
-            'DTL': [1],
-            'EPI': [1],
             'DRAIN': [0, 1, 3],
             'OCC': [1, 2],
+            'SHARED': [0, 1],
         }
 
         # Load template
@@ -108,7 +112,10 @@ class GemmTuner:
 
     @staticmethod
     def config_name(params: Dict[str, int]) -> str:
-        return kc.config_name(dict({'OCC': 1}, **params))
+        c = dict({'OCC': 1, 'SWZ': 1, 'DTL': 1, 'EPI': 1}, **params)
+        if c['KIND'] == 'stream':
+            c['BN'] = 32
+        return kc.config_name(c)
 
     def generate_code(self, params: Dict[str, int]) -> str:
         """Generate code with given parameters"""
@@ -160,17 +167,21 @@ class GemmTuner:
         # Run the benchmark
         return self._run(test_file, params)
 
+    # parameters that mean nothing for a kind: only their first value in the space is kept
+    UNUSED = {'tile': ('NS', 'DRAIN', 'SHARED'), 'mfma16': ('NS', 'SHARED'), 'ring': ('DRAIN', 'OCC', 'SHARED'),
+              'ring16': ('DRAIN', 'OCC', 'SHARED'), 'stream': ('BN', 'WM', 'WN', 'GROUP', 'DRAIN', 'OCC', 'SHARED'),
+              'decode': ('WM', 'WN', 'GROUP', 'DRAIN', 'OCC', 'SHARED'), 'wavek': ('WM', 'WN', 'GROUP', 'DRAIN', 'OCC')}
+
     def is_valid_configuration(self, params: Dict[str, int]) -> bool:
         """Check if a parameter configuration is valid"""
-        c = dict({'OCC': 1}, **params)
-        if c['KIND'] != 'tile' and (c.get('SWZ', 1) != 1 or c.get('DTL', 1) != 1 or c.get('EPI', 1) != 1):
-            return False            # only the two-stage kernel has several load paths and epilogues
-        if c['KIND'] in ('ring', 'ring16') and c.get('OCC', 1) != 1:
-            return False            # the ring kernels fill LDS with one workgroup
-        if c['KIND'] != 'mfma16' and c.get('DRAIN', 0) != 0:
-            return False            # the early drain barrier exists in the 16x16x32 two-stage kernel only
-        if c['KIND'] in ('tile', 'mfma16') and c.get('NS', 4) != self.param_space['NS'][0]:
-            return False            # NS is meaningless for the two-stage kernels: keep one copy
+        c = dict({'OCC': 1, 'SWZ': 1, 'DTL': 1, 'EPI': 1}, **params)
+        for key in self.UNUSED.get(c['KIND'], ()):
+            if key in params and key in self.param_space and params[key] != self.param_space[key][0]:
+                return False        # one copy of the configuration, not one per value of a parameter it ignores
+        if c['KIND'] == 'stream':
+            c['BN'] = 32            # the single-pass decode kernel owns 32 columns per workgroup
+        if c['KIND'] == 'wavek' and not c.get('SHARED'):
+            c.pop('SHARED', None)
         try:
             return kc.is_valid_config(c)
         except KeyError:

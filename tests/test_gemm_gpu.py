@@ -972,23 +972,28 @@ def test_harness_programs(mi):
 
 def test_tuner_rendered_programs_run_and_feed_the_tuner(mi, tmp_path):
     """The tuner's own flow on the GPU (gemm_tuner.py:34-72 of the reference: render -> compile
-    -> run `./test M m N n K k` -> parse the latency line).  The two sample configurations the
-    build rendered from template/matmul_mi355x.hip.jinja (a 16x16x32 kernel with the drain
-    barrier and a 32x32x16 two-per-CU kernel) instantiate their kernels directly, without the
-    library's dispatch.  Each runs an aligned and two ragged shapes against the on-device
+    -> run `./test M m N n K k` -> parse the latency line).  The sample configurations the
+    build rendered from template/matmul_mi355x.hip.jinja -- a 16x16x32 kernel with the drain
+    barrier, a 32x32x16 two-per-CU kernel, and two points of the LDS-stage sweep that the
+    library itself does not compile: a split-K decode kernel with a ring of four slabs and a
+    small-tile kernel with per-wave rings of three stages -- instantiate their kernels directly,
+    without the library's dispatch.  Each runs aligned and ragged shapes against the on-device
     golden; then GemmTuner.tune(prebuilt=True) sweeps them and its outputs are checked."""
     import json
     from h100_gemm_amd import build as lib_build
     from h100_gemm_amd.gemm_tuner import DEFAULT_TEMPLATE, GemmTuner, LATENCY_RE
     bindir = lib_build.TUNER_SAMPLES / "bin"
     tuner = GemmTuner(str(DEFAULT_TEMPLATE), str(tmp_path / "out"), bin_dir=str(bindir),
-                      only=lib_build.TUNER_SAMPLE_CONFIGS, bench_args=("M", "1024", "N", "768", "K", "512", "iters", "20"))
-    names = [tuner.config_name(p) for p in tuner.configurations()]
-    assert len(names) == 2
-    for name in names:
+                      only=lib_build.TUNER_SAMPLE_CONFIGS, bench_args=("M", "128", "N", "768", "K", "512", "iters", "20"))
+    configs = tuner.configurations()
+    names = [tuner.config_name(p) for p in configs]
+    assert len(names) == 4 and {p["KIND"] for p in configs} == {"mfma16", "tile", "decode", "wavek"}
+    shapes = {"decode": (("128", "1024", "1024"), ("100", "516", "1088"), ("37", "8192", "4096")),      # M <= 128, N % 4 == 0, K % 64 == 0
+              None: (("512", "512", "512"), ("257", "515", "77"), ("1000", "300", "1032"))}
+    for p, name in zip(configs, names):
         exe = bindir / name
         assert exe.exists(), f"{exe} is not built (python -m h100_gemm_amd.build)"
-        for shape in (("512", "512", "512"), ("257", "515", "77"), ("1000", "300", "1032")):
+        for shape in shapes.get(p["KIND"], shapes[None]):
             for extra in ([], ["dtype", "fp16"], ["fill", "uniform"]):
                 print(f"case tuner program {name} M N K = {shape} {extra}", flush=True)
                 r = subprocess.run([str(exe), "M", shape[0], "N", shape[1], "K", shape[2], "iters", "3", *extra],
@@ -996,18 +1001,22 @@ def test_tuner_rendered_programs_run_and_feed_the_tuner(mi, tmp_path):
                 assert r.returncode == 0, r.stdout + r.stderr
                 assert f"Shape M={shape[0]}, N={shape[1]}, K={shape[2]}" in r.stdout and "Correct!" in r.stdout
                 assert LATENCY_RE.search(r.stdout) and name in r.stdout, r.stdout
+    # a shape a decode configuration cannot run ends its program with an error, which the tuner scores as a failure
+    decode_exe = bindir / names[[p["KIND"] for p in configs].index("decode")]
+    r = subprocess.run([str(decode_exe), "M", "512", "N", "512", "K", "512", "iters", "3"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0 and "needs M <= 128" in r.stderr
     best_params, best_runtime, results = tuner.tune(prebuilt=True)
-    assert len(results) == 2 and all(r["success"] and 0 < r["runtime"] < 5 for r in results), results
+    assert len(results) == 4 and all(r["success"] and 0 < r["runtime"] < 5 for r in results), results
     assert best_params in lib_build.TUNER_SAMPLE_CONFIGS and best_runtime == min(r["runtime"] for r in results)
     doc = json.loads(sorted((tmp_path / "out").glob("tuning_results_*.json"))[-1].read_text())
     assert set(doc) == {"results", "best_params", "best_runtime", "timestamp"}
     assert set(doc["results"][0]) == {"params", "runtime", "success", "timestamp"}
     assert doc["best_params"] == best_params
     assert f"Best runtime: {best_runtime:.4f} ms" in (tmp_path / "out" / "tuning_summary.txt").read_text()
-    assert f"GROUPM = {best_params['GROUP']};" in (tmp_path / "out" / "best_matmul_mi355x.hip").read_text()
+    assert f"STAGES = {best_params['NS']};" in (tmp_path / "out" / "best_matmul_mi355x.hip").read_text()
     # a configuration that was not compiled scores as a failure and the sweep goes on
     tuner2 = GemmTuner(str(DEFAULT_TEMPLATE), str(tmp_path / "out2"), bin_dir=str(bindir),
-                       only=[dict(lib_build.TUNER_SAMPLE_CONFIGS[0], GROUP=8)] + lib_build.TUNER_SAMPLE_CONFIGS[1:],
+                       only=[dict(lib_build.TUNER_SAMPLE_CONFIGS[0], GROUP=8)] + lib_build.TUNER_SAMPLE_CONFIGS[1:2],
                        bench_args=("M", "512", "N", "512", "K", "512", "iters", "5"))
     bp, br, res = tuner2.tune(prebuilt=True)
     assert [r["success"] for r in res] == [False, True] and bp == lib_build.TUNER_SAMPLE_CONFIGS[1]

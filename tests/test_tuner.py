@@ -110,8 +110,41 @@ def test_default_search_space_is_valid_and_covers_the_shipped_big_kernels():
     t = GemmTuner.__new__(GemmTuner)
     GemmTuner.__init__(t, str(DEFAULT_TEMPLATE), "/tmp/_tuner_space_check")
     cfgs = t.configurations()
-    assert 20 <= len(cfgs) <= 200
-    assert all(kc.is_valid_config(dict(c, OCC=1)) for c in cfgs)
+    assert 20 <= len(cfgs) <= 400
+    assert all(t.is_valid_configuration(c) for c in cfgs)
     names = {t.config_name(c) for c in cfgs}
     assert "r256x256_w2x2_n4_g8" in names and "t256x256_w2x2_s1_g8_o1_d1_e1" in names
     assert LATENCY_RE.search("Average latency (ms) is 0.8057").group(1) == "0.8057"
+
+
+def test_the_grid_sweeps_lds_stages_where_the_depth_is_a_parameter(tmp_path):
+    """MFMA tile, wave layout and LDS stage count (the reference sweeps BLOCKM and STAGES,
+    gemm_tuner.py:17-24): the decode kinds and the small-tile kind appear with several ring
+    depths each, every point is a valid configuration with a name of its own, parameters a kind
+    ignores do not multiply it, and the template renders every kind."""
+    t = GemmTuner(str(DEFAULT_TEMPLATE), str(tmp_path / "out"))
+    assert not {"SWZ", "DTL", "EPI"} & set(t.param_space)            # single-valued knobs are not part of the grid
+    cfgs = t.configurations()
+    names = [t.config_name(c) for c in cfgs]
+    assert len(set(names)) == len(names) > 200
+    by_kind = {}
+    for c in cfgs:
+        by_kind.setdefault(c["KIND"], set()).add(c["NS"])
+    assert by_kind["stream"] >= {2, 3, 4, 5} and by_kind["decode"] == {3, 4, 5} and by_kind["wavek"] >= {1, 2, 3, 4}
+    assert by_kind["tile"] == {4} and by_kind["mfma16"] == {4} and by_kind["ring"] == {4}      # (two-stage kernels: one copy; rings of four)
+    for c in cfgs:
+        full = dict({"OCC": 1, "SWZ": 1, "DTL": 1, "EPI": 1}, **c)
+        if c["KIND"] == "stream":
+            full["BN"] = 32
+        if c["KIND"] == "wavek" and not c["SHARED"]:
+            full.pop("SHARED")
+        assert kc.is_valid_config(full), c
+    # the library's own decode and small-tile configurations are points of this grid
+    for lib in kc.CONFIGS:
+        if lib["KIND"] in ("stream", "decode", "wavek"):
+            assert kc.config_name(lib) in names, kc.config_name(lib)
+    for kind in ("stream", "decode", "wavek"):
+        c = next(c for c in cfgs if c["KIND"] == kind and c["NS"] == 3)
+        src = t.generate_code(c)
+        assert f"#define KERNEL_KIND_{kind.upper()} 1" in src and "static constexpr int STAGES = 3;" in src
+        assert f'"{t.config_name(c)}"' in src
