@@ -158,7 +158,7 @@ TUNER_SAMPLE_CONFIGS = [
     # slabs of B and a small-tile kernel with per-wave rings of three stages (neither depth is
     # among the library's own configurations)
     dict(KIND="decode", BM=128, BN=128, WM=2, WN=2, NS=4, GROUP=4, DRAIN=0, OCC=1, SHARED=0),
-    dict(KIND="wavek", BM=64, BN=64, WM=2, WN=2, NS=3, GROUP=4, DRAIN=0, OCC=1, SHARED=0),
+    dict(KIND="wavek", BM=32, BN=32, WM=2, WN=2, NS=3, GROUP=4, DRAIN=0, OCC=1, SHARED=0),
 ]
 
 

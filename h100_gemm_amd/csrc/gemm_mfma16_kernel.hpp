@@ -100,8 +100,8 @@ __device__ __forceinline__ f32x4_t mfma_16x16x32(u32x4_t a, u32x4_t b, f32x4_t c
 // Only when the header is compiled with -DMI_GEMM_ABLATE (harness/gemm_power.hip does, the
 // library does not) the kernel takes a fourth parameter ABLATE that compiles parts of the K
 // loop out, so that their share of cycles and of power can be read off -- bit 0: no global ->
-// LDS loads after the prologue, bit 1: no LDS fragment reads in the loop, bit 2: no barriers.
-// The results of such a kernel are meaningless.  In the library's build MI_ABLATED is `false`.
+// LDS loads after the prologue, bit 1: no LDS fragment reads in the loop, bit 2: no barriers,
+// bit 3: no epilogue (C is not written).  The results of such a kernel are meaningless.  In the library's build MI_ABLATED is `false`.
 #ifdef MI_GEMM_ABLATE
 #define MI_ABLATED(bits) ((ABLATE & (bits)) != 0)
 template <class Cfg, bool TRACE = false, bool SPLITK = false, int ABLATE = 0>
@@ -572,6 +572,12 @@ gemm_mfma16_kernel(const GemmArgs p) {
     };
     if constexpr (SPLITK) {
         store_partials();
+    } else if constexpr (MI_ABLATED(8)) {
+        // (ablation bit 3: no epilogue at all -- what hiding it completely could gain at most)
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+            for (int j = 0; j < NI; ++j) asm volatile("" :: "a"(acc[i][j]));
     } else {
         if (p.alpha != 1.0f || p.beta != 0.0f) epilogue(std::true_type{});
         else epilogue(std::false_type{});

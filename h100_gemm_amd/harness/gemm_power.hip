@@ -153,6 +153,7 @@ int main(int argc, char** argv) {
         {"no global->LDS loads", launch_variant<1>, 0},
         {"no loads, no fragment reads", launch_variant<3>, 0},
         {"MFMAs only (no loads, reads, barriers)", launch_variant<7>, 0},
+        {"no epilogue (C not written)", launch_variant<8>, 0},
         {"fp16 storage, the bf16 values: full kernel", launch_variant<0, mi::DT_FP16>, 1},
         {"fp16 storage, the bf16 values: MFMAs only", launch_variant<7, mi::DT_FP16>, 1},
         {"fp16 storage, U[-1,1) in fp16: full kernel", launch_variant<0, mi::DT_FP16>, 2},
