@@ -153,7 +153,8 @@ gemm_mfma16_kernel(const GemmArgs p) {
     const int M = p.M, N = p.N;
     const int K = SPLITK ? ((p.K - k0) < p.k_per_split ? (p.K - k0) : p.k_per_split) : p.K / Cfg::KG;
     // K steps: an even number.  The aligned variant is only launched with K % 128 == 0; the
-    // predicated one rounds up and the surplus (part of a) slab is zeroed in LDS.
+    // predicated one rounds up and the surplus (part of a) slab is zeroed in LDS (a slab that
+    // lies past K altogether is still loaded and zeroed, but its step is not run).
     const int KT = EDGE ? ((K + 2 * BK - 1) / (2 * BK)) * 2 : K / BK;
 
     // Descriptors end exactly at the last element of the tile's last valid row: nothing past
@@ -446,7 +447,8 @@ gemm_mfma16_kernel(const GemmArgs p) {
             kt += 2;
         }
         kstep(kt, S0{}, T{}, F{}, T{});
-        kstep(kt + 1, S1{}, F{}, F{}, F{});
+        // the surplus slab of an odd number of 64-deep slabs is all zeros: its step is skipped
+        if ((kt + 1) * BK < K) kstep(kt + 1, S1{}, F{}, F{}, F{});
     }
 
     long long tr_store = 0;
