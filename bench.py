@@ -71,7 +71,7 @@ MEASURED_TRAFFIC_KIB = {
     "unaligned": ("m256x192_w2x2_g4_b3", "gemm_mfma16_kernel_unaligned.md", (130077,), (49670,)),      # 0.317 GB against 0.113 GB algorithmic
     "mlp_up": ("m256x256_w2x2_g4_b3", "gemm_mfma16_kernel_mlp_up.md", (2753369,), (458767,)),          # 6.1 GB against 1.34 GB algorithmic
     "mlp_down": ("m256x256_w2x2_g8_b1", "gemm_mfma16_kernel_mlp_down.md", (2752957,), (131159,)),      # 5.8 GB against 1.07 GB algorithmic
-    "square512": ("k32x32_n2", "gemm_wavek_kernel_square512.md", (1565,), (512,)),                     # 3.7 MB against 1.5 MB algorithmic: a copy of the rows per L2
+    "square512": ("k32x32_s4", "gemm_shared_ring_kernel_square512.md", (1587,), (512,)),                     # 3.7 MB against 1.5 MB algorithmic: a copy of the rows per L2
     "fewtile512": ("k32x32_n2", "gemm_wavek_kernel_fewtile.md", (12317,), (512,)),                     # 25.8 MB against 8.9 MB algorithmic
     "fewtile1024": ("k64x64_n2", "gemm_wavek_kernel_fewtile.md", (24627,), (2048,)),                   # 52.5 MB against 18.9 MB algorithmic
     "skinny64": ("d64x128_n4", "gemm_decode_kernel_skinny128_skinny64.md", (69689, 4114), (8192, 1024)),      # main + reduce kernels

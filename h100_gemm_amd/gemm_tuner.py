@@ -341,6 +341,11 @@ def main(argv=None):
     ap.add_argument("--resume", default=None, help="results JSON of an earlier run to continue from")
     ap.add_argument("--shape", nargs=3, type=int, default=[5120, 5120, 4096], metavar=("M", "N", "K"))
     ap.add_argument("--fill", default=None, choices=["int", "uniform", "normal"])
+    ap.add_argument("--iters", type=int, default=None, help="timed launches per configuration (default: the program's 200)")
+    ap.add_argument("--kinds", default=None,
+                    help="comma-separated kernel kinds to keep of the grid, e.g. stream,decode,wavek (default: all)")
+    ap.add_argument("--bin-dir", default=None, help="where --prebuild puts and --prebuilt finds the programs "
+                                                    "(default: <output-dir>/bin)")
     ap.add_argument("-j", "--jobs", type=int, default=8)
     ap.add_argument("--write-tuned", metavar="FILE", default=None,
                     help="instead of sweeping the template: time the library's compiled candidates for the shapes "
@@ -355,7 +360,16 @@ def main(argv=None):
     bench_args = ["M", str(a.shape[0]), "N", str(a.shape[1]), "K", str(a.shape[2])]
     if a.fill:
         bench_args += ["fill", a.fill]
-    tuner = GemmTuner(str(DEFAULT_TEMPLATE), a.output_dir, bench_args=bench_args, resume_from=a.resume)
+    if a.iters:
+        bench_args += ["iters", str(a.iters)]
+    tuner = GemmTuner(str(DEFAULT_TEMPLATE), a.output_dir, bench_args=bench_args, resume_from=a.resume,
+                      bin_dir=a.bin_dir)
+    if a.kinds:
+        kinds = a.kinds.split(",")
+        unknown = sorted(set(kinds) - set(tuner.param_space['KIND']))
+        if unknown:
+            ap.error(f"unknown kind(s) {unknown}; the grid has {tuner.param_space['KIND']}")
+        tuner.param_space['KIND'] = [k for k in tuner.param_space['KIND'] if k in kinds]
     if a.prebuild:
         built = tuner.prebuild(a.jobs)
         print(f"compiled {sum(built.values())} of {len(built)} configurations into {tuner.bin_dir}")

@@ -11,6 +11,12 @@
 //     dtype <bf16|fp16>  storage type (default bf16; the reference program is fp16)
 //     iters <n>          timed launches (default 200, as in the reference)
 //     check <0|1>        skip / run the comparison (default 1)
+//     rotate <n>         copies of A and B the timed launches take in turn (default 0: one
+//                        when A, B and C together exceed the chip's 256 MB memory-side cache,
+//                        else as many as make the set 512 MiB, at most eight).  That cache
+//                        would otherwise hold a B of 128 MiB from one launch to the next, and
+//                        a timing loop over one buffer would rank the HBM-bound decode
+//                        kernels by how they read the cache, not HBM
 //     fill <int|uniform|normal>  inputs: the reference's integer random_fill (default),
 //                        seeded U[-1,1), or seeded A ~ N(0,1), B ~ N(0,0.02^2); with the
 //                        last two the sums are inexact and the comparison is the bound
@@ -22,8 +28,10 @@
 //                        C[n*M + m] (matmul_utils.cuh:545)         } reads test_epilogue()
 #pragma once
 
+#include <algorithm>
 #include <functional>
 #include <string>
+#include <vector>
 
 #include "gemm_host.hpp"
 
@@ -47,7 +55,7 @@ const int testN = 4096;
 const int testK = 4096;
 
 template <class T>
-int run_test(int M, int N, int K, int config, int iters, bool check, const std::string& fill,
+int run_test(int M, int N, int K, int config, int iters, bool check, int rotate, const std::string& fill,
              const TestLaunchFn& launch, const std::function<std::string(int)>& label) {
     using AType = T;
     using BType = T;
@@ -122,11 +130,31 @@ int run_test(int M, int N, int K, int config, int iters, bool check, const std::
         std::cout << "Correct!\n";
     }
 
+    // the operand copies the timed launches rotate through
+    if (rotate <= 0) {
+        const size_t ab = (shape_numel(AShape) + shape_numel(BShape)) * sizeof(T);
+        const size_t abc = ab + shape_numel(CShape) * sizeof(T);
+        rotate = abc >= ((size_t)256 << 20) ? 1 : (int)std::min<size_t>(8, (((size_t)512 << 20) + ab - 1) / ab);
+    }
+    std::vector<AType*> rA = {dA};
+    std::vector<BType*> rB = {dB};
+    for (int c = 1; c < rotate; ++c) {
+        rA.push_back(alloc_gpu_tensor<AType>(AShape));
+        rB.push_back(alloc_gpu_tensor<BType>(BShape));
+        copy_to_gpu(hA, rA.back(), AShape);
+        copy_to_gpu(hB, rB.back(), BShape);
+    }
+    for (int i = 0; i < rotate; ++i) launch(dt, config, M, N, K, rA[i], rB[i], dC);   // untimed: first touch of every copy
+
     gpu_timer.sync_all();
     gpu_timer.tick();
-    for (int i = 0; i < iters; ++i) launch(dt, config, M, N, K, dA, dB, dC);
+    for (int i = 0; i < iters; ++i) launch(dt, config, M, N, K, rA[i % rotate], rB[i % rotate], dC);
     gpu_timer.tick();
     gpu_timer.sync_all();
+    for (int c = 1; c < rotate; ++c) {
+        free_gpu_tensor(rA[c]);
+        free_gpu_tensor(rB[c]);
+    }
     float latency = gpu_timer.report_last_ms() / float(iters);
     std::cout << "Average latency (ms) is " << latency << "\n";
     const double tflops = 2.0 * M * N * K / (latency * 1e-3) / 1e12;
@@ -147,7 +175,7 @@ inline int test_main(int argc, char** argv, const TestLaunchFn& launch,
                      const std::function<std::string(int)>& label,
                      const std::function<int(const char*)>& parse_config) {
     int M = testM, N = testN, K = testK;
-    int iters = 200, config = MI_CONFIG_AUTO;
+    int iters = 200, config = MI_CONFIG_AUTO, rotate = 0;
     bool check = true;
     std::string dtype = "bf16", fill = "int";
     if (argc > 1) {
@@ -160,6 +188,7 @@ inline int test_main(int argc, char** argv, const TestLaunchFn& launch,
             else if (keys == "K") K = std::atoi(value);
             else if (keys == "iters") iters = std::atoi(value);
             else if (keys == "check") check = std::atoi(value) != 0;
+            else if (keys == "rotate") rotate = std::atoi(value);
             else if (keys == "dtype") dtype = value;
             else if (keys == "fill") fill = value;
             else if (keys == "alpha") test_epilogue().alpha = (float)std::atof(value);
@@ -180,6 +209,6 @@ inline int test_main(int argc, char** argv, const TestLaunchFn& launch,
         return 2;
     }
     std::cout << "Shape M=" << M << ", N=" << N << ", K=" << K << "\n";
-    if (dtype == "fp16") return run_test<half_t>(M, N, K, config, iters, check, fill, launch, label);
-    return run_test<bf16>(M, N, K, config, iters, check, fill, launch, label);
+    if (dtype == "fp16") return run_test<half_t>(M, N, K, config, iters, check, rotate, fill, launch, label);
+    return run_test<bf16>(M, N, K, config, iters, check, rotate, fill, launch, label);
 }

@@ -286,6 +286,9 @@ CONFIGS = [
     _k(64, 64, NS=4, SHARED=1, OCC=2, WK=(1.31, 1.734, 0.1815, 0.0), WK_RAGGED=(1.06, 1.44, 1.31, 1.60), WK_ODD=1.77),
     _k(96, 64, NS=4, SHARED=1, OCC=2, WK=(1.96, 1.90, 0.2313, 0.217), WK_RAGGED=(0.98, 1.32, 1.21, 1.52), WK_ODD=1.72),
     _k(64, 32, NS=4, SHARED=1, OCC=3, WK=(1.54, 1.362, 0.1234, 0.0), WK_RAGGED=(1.20, 1.49, 1.49, 1.64), WK_ODD=1.92),
+    # found by the tuner's sweep of the small-tile kinds at 512^3 (256 tiles, one per CU, eight K
+    # units: too few to split over the waves); no time model, a tuned shape only
+    _k(32, 32, NS=4, SHARED=1, OCC=4),
 ]
 
 assert all(is_valid_config(c) for c in CONFIGS), [config_name(c) for c in CONFIGS if not is_valid_config(c)]
@@ -295,7 +298,9 @@ assert len({config_name(c) for c in CONFIGS}) == len(CONFIGS)
 # the 256x256 family (GROUP 4 / 8 x DRAIN 0 / 1 / 3) at the benchmark shapes: at 8192^3 and
 # N = 28672 the default is level with or ahead of the others; at K = 28672 groups 8 tiles tall
 # with the earlier drain slot are 1.7 % faster (2.426 against 2.468 ms).
-TUNED_SHAPES = {(8192, 8192, 28672): "m256x256_w2x2_g8_b1"}
+# 512^3: the tuner's sweep of the small-tile kinds (32x32 tiles, one per CU: the 2 x 2 wave grid
+# on a shared ring of four stages 3.2 us, K split over the waves 3.6).
+TUNED_SHAPES = {(8192, 8192, 28672): "m256x256_w2x2_g8_b1", (512, 512, 512): "k32x32_s4"}
 assert all(n in {config_name(c) for c in CONFIGS} for n in TUNED_SHAPES.values())
 
 # The kernels the automatic choice for decode shapes names (select_decode_kernel in

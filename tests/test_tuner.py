@@ -148,3 +148,27 @@ def test_the_grid_sweeps_lds_stages_where_the_depth_is_a_parameter(tmp_path):
         src = t.generate_code(c)
         assert f"#define KERNEL_KIND_{kind.upper()} 1" in src and "static constexpr int STAGES = 3;" in src
         assert f'"{t.config_name(c)}"' in src
+
+
+def test_cli_keeps_the_kinds_asked_for(tmp_path, monkeypatch, capsys):
+    """`--kinds` cuts the grid down to some kernel kinds (the decode shapes are swept over the
+    decode and small-tile kinds only); an unknown kind is a usage error."""
+    from h100_gemm_amd import gemm_tuner
+    seen = {}
+
+    def fake_tune(self, prebuilt=False):
+        seen["kinds"] = {c["KIND"] for c in self.configurations()}
+        seen["n"] = len(self.configurations())
+        seen["args"] = list(self.bench_args)
+        seen["bin"] = self.bin_dir
+        return None, float("inf"), []
+
+    monkeypatch.setattr(gemm_tuner.GemmTuner, "tune", fake_tune)
+    rc = gemm_tuner.main(["--output-dir", str(tmp_path / "o"), "--kinds", "stream,decode", "--shape", "64", "8192", "8192",
+                          "--fill", "normal", "--iters", "500", "--bin-dir", str(tmp_path / "b"), "--prebuilt"])
+    assert rc == 0 and seen["kinds"] == {"stream", "decode"} and 40 <= seen["n"] <= 60
+    assert seen["args"] == ["M", "64", "N", "8192", "K", "8192", "fill", "normal", "iters", "500"]
+    assert seen["bin"] == tmp_path / "b"
+    with pytest.raises(SystemExit):
+        gemm_tuner.main(["--kinds", "wgmma"])
+    assert "unknown kind" in capsys.readouterr().err
