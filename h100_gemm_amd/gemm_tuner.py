@@ -342,6 +342,9 @@ def main(argv=None):
     ap.add_argument("--shape", nargs=3, type=int, default=[5120, 5120, 4096], metavar=("M", "N", "K"))
     ap.add_argument("--fill", default=None, choices=["int", "uniform", "normal"])
     ap.add_argument("--iters", type=int, default=None, help="timed launches per configuration (default: the program's 200)")
+    ap.add_argument("--no-check", action="store_true",
+                    help="skip each program's comparison with the on-device golden (large shapes: the golden "
+                         "kernel takes longer than the sweep)")
     ap.add_argument("--kinds", default=None,
                     help="comma-separated kernel kinds to keep of the grid, e.g. stream,decode,wavek (default: all)")
     ap.add_argument("--bin-dir", default=None, help="where --prebuild puts and --prebuilt finds the programs "
@@ -362,6 +365,8 @@ def main(argv=None):
         bench_args += ["fill", a.fill]
     if a.iters:
         bench_args += ["iters", str(a.iters)]
+    if a.no_check:
+        bench_args += ["check", "0"]
     tuner = GemmTuner(str(DEFAULT_TEMPLATE), a.output_dir, bench_args=bench_args, resume_from=a.resume,
                       bin_dir=a.bin_dir)
     if a.kinds:

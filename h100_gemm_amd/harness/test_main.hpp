@@ -11,11 +11,12 @@
 //     dtype <bf16|fp16>  storage type (default bf16; the reference program is fp16)
 //     iters <n>          timed launches (default 200, as in the reference)
 //     check <0|1>        skip / run the comparison (default 1)
-//     rotate <n>         copies of A and B the timed launches take in turn (default 0: one
-//                        when A, B and C together exceed the chip's 256 MB memory-side cache,
-//                        else as many as make the set 512 MiB, at most eight).  That cache
-//                        would otherwise hold a B of 128 MiB from one launch to the next, and
-//                        a timing loop over one buffer would rank the HBM-bound decode
+//     rotate <n>         copies of A and B the timed launches take in turn.  Default 0: for
+//                        a shape that HBM bounds (fewer flops per byte than the chip's peaks
+//                        stand for) and whose A, B and C together fit the 256 MB memory-side
+//                        cache, as many as make the set 512 MiB, at most eight; else one.
+//                        That cache would otherwise hold a B of 128 MiB from one launch to
+//                        the next, and a timing loop over one buffer would rank the decode
 //                        kernels by how they read the cache, not HBM
 //     fill <int|uniform|normal>  inputs: the reference's integer random_fill (default),
 //                        seeded U[-1,1), or seeded A ~ N(0,1), B ~ N(0,0.02^2); with the
@@ -134,7 +135,8 @@ int run_test(int M, int N, int K, int config, int iters, bool check, int rotate,
     if (rotate <= 0) {
         const size_t ab = (shape_numel(AShape) + shape_numel(BShape)) * sizeof(T);
         const size_t abc = ab + shape_numel(CShape) * sizeof(T);
-        rotate = abc >= ((size_t)256 << 20) ? 1 : (int)std::min<size_t>(8, (((size_t)512 << 20) + ab - 1) / ab);
+        const bool hbm_bound = 2.0 * M * N * K / (double)abc < 2.5e15 / 8.0e12;       // flops per byte below the chip's ridge
+        rotate = !hbm_bound || abc >= ((size_t)256 << 20) ? 1 : (int)std::min<size_t>(8, (((size_t)512 << 20) + ab - 1) / ab);
     }
     std::vector<AType*> rA = {dA};
     std::vector<BType*> rB = {dB};

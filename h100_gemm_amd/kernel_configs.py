@@ -23,7 +23,9 @@ template takes (matmul_h100.cu.jinja:9-14) -- re-cast for CDNA4:
              same tile and add their accumulators through LDS (K % 256 == 0; tiles alone on a CU)
     DRAIN    (mfma16, optional) d > 0: a second barrier early in each K step (4*d MFMAs after the
              fragment reads) frees the current LDS stage, so the next loads are spread over most
-             of the step instead of its second half
+             of the step instead of its second half; EDRAIN (optional): the predicated variant's
+             slot where it differs (its loads from unaligned rows arrive later: the earlier slot
+             is 2 % ahead at 4095 x 6143 x 3073, the later one on aligned shapes)
     EWM, EWN (optional) wave grid of the predicated twin when it differs from WM, WN (the
              register-staged predicated kernel runs best with eight waves)
     EFF      (optional) per-CU throughput relative to the 256x256 tile, measured at 8192^3;
@@ -158,8 +160,8 @@ def is_valid_config(c: dict) -> bool:
         tn = c["BN"] // c["WN"]
         if tn < 32 or (c["KIND"] == "ring16" and tn & (tn - 1)):   # ring16: C staging needs a power-of-two row
             return False
-        if c["KIND"] == "mfma16" and c.get("DRAIN", 0):
-            sa = mi16 + ni16 + 4 * c["DRAIN"]
+        for d in {c.get("DRAIN", 0), c.get("EDRAIN", c.get("DRAIN", 0))} - {0} if c["KIND"] == "mfma16" else ():
+            sa = mi16 + ni16 + 4 * d
             if sa + 1 >= mi16 * ni16 or (2 * mi16 * ni16 - 5 - sa) // l < 1:
                 return False
         if mi16 + ni16 + l > mi16 * ni16:
@@ -197,8 +199,10 @@ def _r(BM, BN, WM, WN, NS=4, GROUP=8):
     return dict(KIND="ring", BM=BM, BN=BN, WM=WM, WN=WN, NS=NS, GROUP=GROUP)
 
 
-def _m(BM, BN, WM, WN, GROUP=4, EFF=None, DRAIN=0, OCC=1, EFF_E=None, KG=1):
+def _m(BM, BN, WM, WN, GROUP=4, EFF=None, DRAIN=0, OCC=1, EFF_E=None, KG=1, EDRAIN=None):
     c = dict(KIND="mfma16", BM=BM, BN=BN, WM=WM, WN=WN, GROUP=GROUP)
+    if EDRAIN is not None:
+        c["EDRAIN"] = EDRAIN        # drain slot of the predicated variant, where it differs
     if KG != 1:
         c["KG"] = KG
     if EFF_E is not None:
@@ -257,8 +261,8 @@ CONFIGS = [
     _r(256, 256, 2, 2),
     _r(256, 256, 2, 4),
     _m(256, 256, 2, 2),
-    _m(256, 256, 2, 2, DRAIN=3, EFF=1.0, EFF_E=0.82),
-    _m(256, 192, 2, 2, DRAIN=3, EFF=0.89, EFF_E=0.90),
+    _m(256, 256, 2, 2, DRAIN=3, EDRAIN=1, EFF=1.0, EFF_E=0.86),
+    _m(256, 192, 2, 2, DRAIN=3, EDRAIN=1, EFF=0.89, EFF_E=0.92),
     _m(128, 256, 2, 2, DRAIN=1, EFF=0.84, EFF_E=0.80),
     _m(256, 128, 2, 2, DRAIN=1, EFF=0.845, EFF_E=0.80),
     _m(128, 128, 2, 2, DRAIN=1, OCC=2, EFF=0.78, EFF_E=0.74),
