@@ -55,7 +55,7 @@ LATENCY_RE = re.compile(r"Average latency \(ms\) is ([\d.]+(?:e[-+]?\d+)?)")
 def default_compile_command(src: str, exe: str) -> List[str]:
     return [os.environ.get("HIPCC", "/opt/rocm/bin/hipcc"), "--offload-arch=gfx950", "-O3", "-std=c++17",
             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-            "-Wno-unused-command-line-argument", f"-I{PKG / 'csrc'}", f"-I{PKG / 'harness'}",
+            "-Wno-unused-command-line-argument", "-pthread", f"-I{PKG / 'csrc'}", f"-I{PKG / 'harness'}",
             src, "-o", exe, f"-L{PKG / 'lib'}", "-lmi_gemm", f"-Wl,-rpath,{PKG / 'lib'}"]
 
 

@@ -17,6 +17,7 @@
 // message with file:line and exit(EXIT_FAILURE) (common.h:29-37, matmul_h100_optimal.cu:21-28).
 #pragma once
 
+#include <algorithm>
 #include <cassert>
 #include <chrono>
 #include <cmath>
@@ -29,6 +30,7 @@
 #include <numeric>
 #include <random>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "../../include/mi_gemm.h"
@@ -234,27 +236,40 @@ inline uint64_t mi_mix64(uint64_t z) {
 inline uint64_t mi_rng_u64(uint64_t seed, uint64_t stream, uint64_t index) {
     return mi_mix64(mi_mix64(seed ^ (stream * 0xd1342543de82ef95ull)) + index);
 }
+// fn(begin, end) over [0, length) in contiguous pieces on up to 16 host threads (the fills below
+// are pure functions of the index, so the result does not depend on the split)
+template <class Fn>
+void for_index_ranges(size_t length, Fn fn) {
+    const unsigned hw = std::thread::hardware_concurrency();
+    const size_t nt = std::min<size_t>(std::min<size_t>(hw ? hw : 1, 16), std::max<size_t>(1, length >> 20));
+    if (nt <= 1) return fn((size_t)0, length);
+    std::vector<std::thread> pool;
+    for (size_t t = 0; t < nt; ++t) pool.emplace_back(fn, length * t / nt, length * (t + 1) / nt);
+    for (auto& th : pool) th.join();
+}
 // i.i.d. uniform on the 2^-23 grid of [-1, 1), rounded to the storage type.
 template <class DType>
 void uniform_fill(DType* tensor, std::vector<int> shape, uint64_t seed, uint64_t stream) {
-    const size_t length = shape_numel(shape);
-    for (size_t i = 0; i < length; ++i) {
-        const float u = (float)(mi_rng_u64(seed, stream, i) >> 40) * (1.0f / 16777216.0f);
-        tensor[i] = DType(2.0f * u - 1.0f);
-    }
+    for_index_ranges(shape_numel(shape), [=](size_t b, size_t e) {
+        for (size_t i = b; i < e; ++i) {
+            const float u = (float)(mi_rng_u64(seed, stream, i) >> 40) * (1.0f / 16777216.0f);
+            tensor[i] = DType(2.0f * u - 1.0f);
+        }
+    });
 }
 // i.i.d. N(0, sigma^2) by Box-Muller in double, rounded once to the storage type.
 template <class DType>
 void normal_fill(DType* tensor, std::vector<int> shape, uint64_t seed, uint64_t stream,
                  float sigma = 1.0f) {
-    const size_t length = shape_numel(shape);
-    for (size_t i = 0; i < length; ++i) {
-        const uint64_t r = mi_rng_u64(seed, stream, i);
-        const double u1 = ((double)(r >> 40) + 1.0) * (1.0 / 16777216.0);
-        const double u2 = (double)(r & 0xffffffull) * (1.0 / 16777216.0);
-        const double z = std::sqrt(-2.0 * std::log(u1)) * std::cos(6.283185307179586476925 * u2);
-        tensor[i] = DType((float)(z * (double)sigma));
-    }
+    for_index_ranges(shape_numel(shape), [=](size_t b, size_t e) {
+        for (size_t i = b; i < e; ++i) {
+            const uint64_t r = mi_rng_u64(seed, stream, i);
+            const double u1 = ((double)(r >> 40) + 1.0) * (1.0 / 16777216.0);
+            const double u2 = (double)(r & 0xffffffull) * (1.0 / 16777216.0);
+            const double z = std::sqrt(-2.0 * std::log(u1)) * std::cos(6.283185307179586476925 * u2);
+            tensor[i] = DType((float)(z * (double)sigma));
+        }
+    });
 }
 
 template <class DType>
