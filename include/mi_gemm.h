@@ -81,7 +81,9 @@ int mi_gemm_epilogue(int config, int dtype, int M, int N, int K, const void* A, 
  * mi_gemm_release_workspace gives the stream's buffers back.  At most 16 streams per device
  * hold a buffer: a further stream waits for the device to go idle (hipDeviceSynchronize) and
  * takes over the smallest entry, so a process that keeps creating streams does not keep
- * growing.  A stream under capture that has no large enough buffer yet runs the launch unsplit;
+ * growing (a graph captured from split-K launches on the stream that loses its entry must not
+ * be replayed afterwards, as after a release: captured work that shares a process with more
+ * than 16 GEMM streams should bring its own workspace).  A stream under capture that has no large enough buffer yet runs the launch unsplit;
  * a first or a growing use calls hipMalloc, which must not happen while ANY thread captures
  * in hipStreamCaptureModeGlobal: reserve beforehand (mi_gemm_reserve_workspace) or use
  * mi_gemm_epilogue_ws / mi_gemm_bf16_noalloc there.  The reference's launchers allocate
