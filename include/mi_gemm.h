@@ -113,7 +113,7 @@ size_t mi_gemm_library_workspace_bytes(void);
 /* Bytes of workspace the library's choice of kernel wants for this call (0 when the shape
  * does not run split-K).  An upper bound: the largest need over the pointer alignments a
  * launch can meet and over the two parts of a shape whose rows the automatic choice cuts
- * (2248 x 8192 x 28672: 210.75 MiB for the uncut split of an unaligned call, 25 MiB for the
+ * (2248 x 8192 x 28672: 140.5 MiB for the uncut split of an unaligned call, 25 MiB for the
  * aligned call, which is cut at 2048 rows). */
 size_t mi_gemm_workspace_bytes(int config, int dtype, int M, int N, int K, int c_layout);
 

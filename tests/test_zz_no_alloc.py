@@ -67,12 +67,13 @@ def test_noalloc_entry_point_refuses_what_does_not_fit(mi, orc):
 
 
 def test_noalloc_entry_point_refuses_a_cut_shape_before_it_writes_anything(mi, orc):
-    """A large ragged shape that the automatic choice runs as two GEMMs (the first 2048 rows,
-    then the rest) and whose second part would need more partial sums than the array holds:
-    the call is refused before the first part is launched, so C is untouched."""
+    """A large ragged shape that the automatic choice runs as two GEMMs (the first 4096 rows,
+    then the 200 left) and whose second part would need more partial sums than the array holds
+    (four pieces of 200 x 12288 fp32: 37.5 MiB): the call is refused before the first part is
+    launched, so C is untouched."""
     L = mi._lib.load()
-    M, N, K = 2298, 8192, 32768
-    assert mi.row_cut(M, N, K) > 0
+    M, N, K = 4296, 12288, 16384
+    assert mi.row_cut(M, N, K) == 4096 and mi.workspace_bytes(M, N, K) > 32 << 20
     dA, dB, dC = mi.DeviceBuffer(M * K * 2), mi.DeviceBuffer(N * K * 2), mi.DeviceBuffer(M * N * 2)
     dA.fill_bytes(0)
     dB.fill_bytes(0)
