@@ -152,7 +152,7 @@ def build(jobs: int | None = None, force: bool = False, verbose: bool = True) ->
 # dispatch.  Built here, where hipcc runs without a GPU, so that the GPU tests only run them.
 TUNER_SAMPLES = PKG / "harness" / "tuner_samples"
 TUNER_SAMPLE_CONFIGS = [
-    dict(KIND="mfma16", BM=256, BN=256, WM=2, WN=2, NS=4, SWZ=1, GROUP=4, DTL=1, EPI=1, DRAIN=3, OCC=1),
+    dict(KIND="mfma16", BM=256, BN=256, WM=2, WN=2, NS=4, SWZ=1, GROUP=4, DTL=1, EPI=1, DRAIN=3, EDRAIN=1, OCC=1),
     dict(KIND="tile", BM=128, BN=128, WM=2, WN=2, NS=4, SWZ=1, GROUP=8, DTL=1, EPI=1, DRAIN=0, OCC=2),
     # kinds whose LDS stage count the tuner sweeps: a split-K decode kernel with a ring of four
     # slabs of B and a small-tile kernel with per-wave rings of three stages (neither depth is
