@@ -271,8 +271,8 @@ CONFIGS = [
     _m(256, 256, 2, 4),
     _q(256, 256, 4, 2),
     _q(256, 256, 2, 2),
-    _s(16, 5),
-    _s(32, 4),
+    _s(16, 3),
+    _s(32, 3),
     _s(64, 3),
     _m(256, 256, 2, 2, GROUP=8, DRAIN=1),
     _m(192, 192, 2, 2, DRAIN=1, EFF=0.80, EFF_E=0.91),
@@ -310,6 +310,6 @@ assert all(n in {config_name(c) for c in CONFIGS} for n in TUNED_SHAPES.values()
 
 # The kernels the automatic choice for decode shapes names (select_decode_kernel in
 # template/kernel_table.hpp.jinja, where the thresholds and the measurements behind them are).
-DECODE_KERNELS = {"stream16": "s16x32_n5", "stream32": "s32x32_n4", "stream64": "s64x32_n3",
+DECODE_KERNELS = {"stream16": "s16x32_n3", "stream32": "s32x32_n3", "stream64": "s64x32_n3",
                   "decode64": "d64x128_n4", "decode128": "d128x128_n3", "tile128x256": "m128x256_w2x2_g4_b1"}
 assert all(n in {config_name(c) for c in CONFIGS} for n in DECODE_KERNELS.values())

@@ -156,7 +156,7 @@ int mi_reference_gpu_gemm(int dtype, int M, int N, int K, const void* A, const v
 int mi_gemm_num_configs(void);
 /* Human-readable name, e.g. "m256x256_w2x2_g4_b3" (16x16x32-MFMA kernel, the default),
  * "t128x128_w2x2_s1_g8_o2_d1_e1" (32x32x16-MFMA kernel), "r256x256_w2x2_n4_g8" (LDS-ring
- * kernel), "s16x32_n5" / "d128x128_n3" (single-pass / split-K decode kernels), "k64x64_n2" /
+ * kernel), "s16x32_n3" / "d128x128_n3" (single-pass / split-K decode kernels), "k64x64_n2" /
  * "k96x96_s4" (small tiles for outputs of few tiles: K split over the waves of a workgroup /
  * the waves sharing one ring of LDS stages); NULL if out of range. */
 const char* mi_gemm_config_name(int config);
