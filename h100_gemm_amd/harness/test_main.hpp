@@ -144,6 +144,7 @@ int run_test(int M, int N, int K, int config, int iters, bool check, int rotate,
         const bool hbm_bound = 2.0 * M * N * K / (double)abc < 2.5e15 / 8.0e12;       // flops per byte below the chip's ridge
         rotate = !hbm_bound || abc >= ((size_t)256 << 20) ? 1 : (int)std::min<size_t>(8, (((size_t)512 << 20) + ab - 1) / ab);
     }
+    if (rotate > 1) std::cout << "Timing over " << rotate << " copies of A and B in turn\n";
     std::vector<AType*> rA = {dA};
     std::vector<BType*> rB = {dB};
     for (int c = 1; c < rotate; ++c) {

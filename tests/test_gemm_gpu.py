@@ -962,6 +962,16 @@ def test_harness_programs(mi):
     assert r.returncode == 0, r.stdout + r.stderr
     assert "Shape M=640, N=384, K=512" in r.stdout and "Correct!" in r.stdout
     assert re.search(r"Average latency \(ms\) is ([\d.]+)", r.stdout)        # the tuner's regex
+    # an HBM-bound shape whose operands would fit the memory-side cache is timed over several
+    # copies of A and B by default (64 x 4096 x 4096: 32.5 MiB a set -> 8 copies), `rotate` overrides
+    r = subprocess.run([str(h / "test"), "M", "64", "N", "4096", "K", "4096", "iters", "20"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0 and "Correct!" in r.stdout and "Timing over 8 copies of A and B in turn" in r.stdout, r.stdout + r.stderr
+    r = subprocess.run([str(h / "test"), "M", "64", "N", "4096", "K", "4096", "iters", "20", "rotate", "3"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0 and "Timing over 3 copies of A and B in turn" in r.stdout, r.stdout + r.stderr
+    assert "Timing over" not in subprocess.run([str(h / "test"), "M", "640", "N", "384", "K", "512", "iters", "5", "rotate", "1"],
+                                               capture_output=True, text=True, timeout=120).stdout
     r = subprocess.run([str(h / "test"), "M", "333", "N", "129", "K", "77", "iters", "2",
                         "dtype", "fp16"], capture_output=True, text=True, timeout=120)
     assert r.returncode == 0 and "Correct!" in r.stdout, r.stdout + r.stderr
