@@ -526,9 +526,10 @@ gemm_mfma16_kernel(const GemmArgs p) {
         };
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");   // all waves done with the last stage
         unsigned char* stg = lds + wave * (TM * TN * 2);
-        // In pieces of 32 rows (where the row layout allows): the stores of one piece drain
-        // while the next is converted, instead of 128 KB per CU queueing up at once.
-        constexpr int CH_ROWS = (POW2 && TM % 32 == 0 && 32 % (64 / CPR) == 0) ? 32 : TM;
+        // In pieces of 32 rows (where they are whole numbers of 64-lane store instructions): the
+        // stores of one piece drain while the next is converted, instead of 128 KB per CU queueing
+        // up at once.
+        constexpr int CH_ROWS = (TM % 32 == 0 && (32 * CPR) % 64 == 0) ? 32 : TM;
 #pragma unroll
         for (int c = 0; c < TM / CH_ROWS; ++c) {
 #pragma unroll
