@@ -290,7 +290,7 @@ CONFIGS = [
     _k(64, 64, NS=4, SHARED=1, OCC=2, WK=(1.31, 1.734, 0.1815, 0.0), WK_RAGGED=(1.06, 1.44, 1.31, 1.60), WK_ODD=1.77),
     _k(96, 64, NS=4, SHARED=1, OCC=2, WK=(1.96, 1.90, 0.2313, 0.217), WK_RAGGED=(0.98, 1.32, 1.21, 1.52), WK_ODD=1.72),
     _k(64, 32, NS=4, SHARED=1, OCC=3, WK=(1.54, 1.362, 0.1234, 0.0), WK_RAGGED=(1.20, 1.49, 1.49, 1.64), WK_ODD=1.92),
-    _m(192, 256, 2, 2, DRAIN=3, EDRAIN=1, EFF=0.89, EFF_E=0.92),
+    _m(192, 256, 2, 2, DRAIN=1, EFF=0.89, EFF_E=0.92),
     # found by the tuner's sweep of the small-tile kinds at 512^3 (256 tiles, one per CU, eight K
     # units: too few to split over the waves); no time model, a tuned shape only
     _k(32, 32, NS=4, SHARED=1, OCC=4),
